@@ -1,0 +1,150 @@
+/*
+ * torchex_scatter.h -- C ABI of the MI355X (gfx950) voxel scatter-reduction
+ * library, libtorchex_scatter.so.
+ *
+ * Plain C: device pointers, 64-bit sizes, an opaque stream handle
+ * (a hipStream_t passed as void*; NULL = the null stream) and an int status.
+ * No torch type crosses this line.  The library allocates no device memory:
+ * every buffer, workspaces included, is owned by the caller.  Calls are
+ * asynchronous on `stream` and re-entrant (no global state).
+ *
+ * Each entry point names the reference interface it stands in for
+ * (paths relative to the TorchEx tree).
+ *
+ * Data layout
+ *   feats      [N, C]   row-major contiguous, dtype fp32 / fp16 / bf16
+ *   unq_inv    [N]      int32 voxel id of every row, any order, ids in [0, U)
+ *   preSum     [U+1]    int32 CSR offsets: rows of voxel u occupy sorted
+ *                       positions preSum[u] .. preSum[u+1]-1
+ *   perm       [N]      int32 row id at each sorted position (stable: ascending
+ *                       row inside a voxel); NULL when unq_inv is already
+ *                       non-decreasing (position == row)
+ *   seg        [N]      int32 voxel id at each sorted position, bit 31 set when
+ *                       the voxel is "special" (see below)
+ *   slot_of    [U]      int32 slot of a special voxel in heavy_ids/scratch, else -1
+ *   heavy_ids  [>=n_special] int32 voxel id per slot
+ *   scratch    [n_special * C] 8-byte cells.  MUST BE ZERO ON ENTRY to
+ *                       txs_scatter_forward and is zero again when the call's
+ *                       kernels have finished.
+ *   out        [U, C]   dtype of feats;  arg [U, C] int32 (row index into feats)
+ *
+ * Special voxels: a voxel with more than `heavy_threshold` rows is reduced by
+ * many wavefronts whose partials meet in `scratch` through atomics (fp32
+ * atomic add for sum/mean, 64-bit atomic max on a packed value|row word for
+ * max); a voxel with zero rows is special too so that it still gets an output
+ * row.  All other voxels are reduced in registers by one group of lanes and
+ * written once.
+ */
+#ifndef TORCHEX_SCATTER_H
+#define TORCHEX_SCATTER_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { TXS_OK = 0, TXS_ERR_INVALID_ARG = 1, TXS_ERR_LAUNCH = 2, TXS_ERR_UNSUPPORTED = 3 };
+enum { TXS_F32 = 0, TXS_F16 = 1, TXS_BF16 = 2 };
+enum { TXS_SUM = 0, TXS_MEAN = 1, TXS_MAX = 2 };
+
+/* Slots of the int32[TXS_STATS_LEN] device array the plan functions fill. */
+enum {
+    TXS_STAT_UNSORTED = 0,     /* 1 if unq_inv[i] > unq_inv[i+1] for some i */
+    TXS_STAT_OUT_OF_RANGE = 1, /* 1 if some id is outside [0, U) */
+    TXS_STAT_MAX_CNT = 2,      /* largest voxel population */
+    TXS_STAT_NUM_SPECIAL = 3,  /* number of special voxels (heavy or empty) */
+    TXS_STAT_NUM_EMPTY = 4,    /* number of voxels with zero rows */
+    TXS_STATS_LEN = 8
+};
+
+/* Library ABI version; bumped when a signature changes. */
+int txs_abi_version(void);
+
+/* Human-readable text for a status code. */
+const char *txs_status_string(int status);
+
+/* Default population above which a voxel is reduced through atomics, and the
+ * number of sorted positions one lane group walks. */
+int txs_default_heavy_threshold(void);
+int txs_chunk_rows(void);
+
+/* ---- index preparation (what ScatterData.__init__ computes) --------------- */
+
+/* Replaces getPreSum_launcher (torchex/src/scatter/scatter.cpp:18, kernel
+ * scatter_kernel.cu:85-100): CSR offsets from the run boundaries of a SORTED
+ * unq_inv.  preSum has `num_presum` entries and must be zero-filled by the
+ * caller (torchex/operator_py/scatter_op.py:126); writes outside it are
+ * dropped. */
+int txs_get_presum(const int32_t *unq_inv, int32_t *preSum, int64_t num_total,
+                   int64_t num_presum, void *stream);
+
+/* Exact histogram of unq_inv plus order / range checks.  Extends
+ * ScatterData.__init__ (scatter_op.py:13-21) to unsorted input.
+ * counts [U] and stats [TXS_STATS_LEN] are zeroed by the call. */
+int txs_plan_count(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
+                   int32_t *counts, int32_t *stats, void *stream);
+
+/* preSum = [0, cumsum(counts)], the special-voxel table and max_cnt.
+ * scan_ws: int32 workspace of txs_scan_workspace_len(num_unq) entries.
+ * heavy_ids must hold num_unq entries (only the first NUM_SPECIAL are used).
+ * For sorted input preSum equals what txs_get_presum produces. */
+int txs_plan_offsets(const int32_t *counts, int64_t num_unq, int32_t heavy_threshold,
+                     int32_t *preSum, int32_t *slot_of, int32_t *heavy_ids, int32_t *stats,
+                     int32_t *scan_ws, void *stream);
+int64_t txs_scan_workspace_len(int64_t n);
+
+/* Stable sort of row ids by voxel id (LSD radix, 3-kernel passes, no
+ * inter-block spinning): fills perm and seg.  sort_ws: int32 workspace of
+ * txs_sort_workspace_len(num_total, num_unq) entries. */
+int txs_plan_sort(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
+                  const int32_t *slot_of, int32_t *perm, int32_t *seg, int32_t *sort_ws,
+                  void *stream);
+int64_t txs_sort_workspace_len(int64_t num_total, int64_t num_unq);
+
+/* seg for input that is already sorted (perm == NULL): seg[j] = unq_inv[j]
+ * with the special bit from slot_of. */
+int txs_plan_seg_sorted(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
+                        const int32_t *slot_of, int32_t *seg, void *stream);
+
+/* counts from CSR offsets, for callers that hold only preSum (the reference's
+ * scatter_ext.sum / scatter_ext.max argument lists, scatter.cpp:20-53), and
+ * seg by binary search of each position in preSum. */
+int txs_counts_from_presum(const int32_t *preSum, int64_t num_unq, int32_t *counts,
+                           int32_t *stats, void *stream);
+int txs_plan_seg_from_presum(const int32_t *preSum, int64_t num_total, int64_t num_unq,
+                             const int32_t *slot_of, int32_t *seg, void *stream);
+
+/* ---- the hot path --------------------------------------------------------- */
+
+/* Forward reduction.  Replaces scatter_sum_launcher / scatter_max_launcher
+ * (scatter.cpp:12-16, kernels scatter_kernel.cu:102-171) and fuses the divide
+ * of ScatterMeanFunction.forward (scatter_op.py:69) for op == TXS_MEAN.
+ *   op TXS_SUM / TXS_MEAN: arg is ignored (may be NULL); fp32 accumulation.
+ *   op TXS_MAX: out = max, arg = smallest row index attaining it; NaN never
+ *     wins; a voxel with no non-NaN entry (or no rows) gets the lowest finite
+ *     value of the dtype and arg = -1 (the reference's (-FLT_MAX, -1) init,
+ *     scatter_kernel.cu:139-140).
+ * out (and arg) need no initialisation: every element is written.
+ * scratch may be NULL when num_special == 0. */
+int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *perm,
+                        const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
+                        const int32_t *heavy_ids, int64_t num_special, void *scratch,
+                        void *out, int32_t *arg, int64_t num_total, int64_t channel,
+                        int64_t num_unq, void *stream);
+
+/* Backward as one gather pass over the sorted positions.  Replaces the ATen
+ * ops of ScatterSumFunction.backward (scatter_op.py:47-50: g[unq_inv]),
+ * ScatterMeanFunction.backward (:74-78: (g / unq_cnts)[unq_inv]) and the
+ * intended ScatterMaxFunction.backward (:106-111: zeros.scatter_(0, arg, g),
+ * i.e. g_in[i,c] = g[u,c] if arg[u,c] == i else 0).
+ * g_in [N, C] needs no initialisation.  arg is read only for TXS_MAX. */
+int txs_scatter_backward(int op, int dtype, const void *grad_out, const int32_t *arg,
+                         const int32_t *perm, const int32_t *seg, const int32_t *preSum,
+                         void *grad_in, int64_t num_total, int64_t channel, int64_t num_unq,
+                         void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TORCHEX_SCATTER_H */

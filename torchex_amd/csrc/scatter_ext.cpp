@@ -1,0 +1,282 @@
+// scatter_ext: PyTorch-ROCm host glue for the voxel scatter path.
+//
+// Takes the place of torchex/src/scatter/scatter.cpp.  The three functions of
+// the reference module keep their names and positional signatures
+// (scatter.cpp:66-70: sum, max, getPreSum; outputs caller-allocated and written
+// in place); the plan/forward/backward functions are what the Python wrappers
+// in torchex_amd/scatter_op.py use.  All device work goes through the C ABI of
+// libtorchex_scatter.so (include/torchex_scatter.h): this file only validates
+// tensors, allocates through the torch caching allocator, picks the current HIP
+// stream and device, and turns status codes into exceptions.
+
+#include <torch/extension.h>
+
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include <optional>
+#include <tuple>
+#include <vector>
+
+#include "torchex_scatter.h"
+
+namespace {
+
+using at::Tensor;
+using OptTensor = std::optional<Tensor>;
+
+void check_dev(const Tensor &x, const char *name) {
+    // same two conditions as CHECK_INPUT in scatter.cpp:4-10
+    TORCH_CHECK(x.device().is_cuda(), name, " must be a GPU tensor");
+    TORCH_CHECK(x.is_contiguous(), name, " must be contiguous");
+}
+
+void check_i32(const Tensor &x, const char *name) {
+    check_dev(x, name);
+    TORCH_CHECK(x.scalar_type() == at::kInt, name, " must be int32, got ", x.scalar_type());
+}
+
+int dtype_code(const Tensor &x, const char *name) {
+    switch (x.scalar_type()) {
+        case at::kFloat: return TXS_F32;
+        case at::kHalf: return TXS_F16;
+        case at::kBFloat16: return TXS_BF16;
+        default: TORCH_CHECK(false, name, " must be float32, float16 or bfloat16, got ", x.scalar_type());
+    }
+    return -1;
+}
+
+void check_status(int st, const char *what) {
+    TORCH_CHECK(st == TXS_OK, "torchex scatter: ", what, " failed: ", txs_status_string(st));
+}
+
+void *cur_stream(const Tensor &x) {
+    return (void *)c10::hip::getCurrentHIPStream(x.device().index()).stream();
+}
+
+const int32_t *i32p(const Tensor &x) { return x.numel() ? x.data_ptr<int32_t>() : nullptr; }
+int32_t *i32w(Tensor &x) { return x.numel() ? x.data_ptr<int32_t>() : nullptr; }
+const int32_t *opt_i32p(const OptTensor &x) { return (x.has_value() && x->defined()) ? i32p(*x) : nullptr; }
+
+Tensor empty_i32(int64_t n, const Tensor &like) {
+    return at::empty({n}, like.options().dtype(at::kInt));
+}
+
+std::vector<int64_t> read_stats(const Tensor &stats) {
+    Tensor h = stats.cpu();  // the one host synchronisation of index preparation
+    std::vector<int64_t> v(TXS_STATS_LEN);
+    for (int i = 0; i < TXS_STATS_LEN; ++i) v[i] = h.data_ptr<int32_t>()[i];
+    return v;
+}
+
+// counts -> preSum, special table, stats (shared tail of both plan builders)
+struct Offsets {
+    Tensor preSum, slot_of, heavy_ids;
+};
+
+Offsets plan_offsets(const Tensor &counts, int64_t U, int64_t heavy_threshold, Tensor &stats) {
+    Offsets o;
+    o.preSum = empty_i32(U + 1, counts);
+    o.slot_of = empty_i32(U, counts);
+    o.heavy_ids = empty_i32(U, counts);
+    Tensor ws = empty_i32(txs_scan_workspace_len(U), counts);
+    check_status(txs_plan_offsets(i32p(counts), U, (int32_t)heavy_threshold, i32w(o.preSum),
+                                  i32w(o.slot_of), i32w(o.heavy_ids), i32w(stats), i32w(ws),
+                                  cur_stream(counts)),
+                 "plan_offsets");
+    return o;
+}
+
+// ScatterData index preparation for an unq_inv in any order
+// (extends torchex/operator_py/scatter_op.py:13-21).
+// returns (preSum, perm | None, seg, slot_of, heavy_ids, stats)
+std::tuple<Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>> build_plan(
+    const Tensor &unq_inv, int64_t num_unq, int64_t heavy_threshold) {
+    check_i32(unq_inv, "unq_inv");
+    TORCH_CHECK(unq_inv.dim() == 1, "unq_inv must be 1-D");
+    TORCH_CHECK(num_unq >= 0, "num_unq must be non-negative");
+    c10::hip::HIPGuard guard(unq_inv.device());
+    const int64_t N = unq_inv.numel(), U = num_unq;
+    Tensor counts = empty_i32(U, unq_inv);
+    Tensor stats = empty_i32(TXS_STATS_LEN, unq_inv);
+    void *st = cur_stream(unq_inv);
+    check_status(txs_plan_count(i32p(unq_inv), N, U, i32w(counts), i32w(stats), st), "plan_count");
+    Offsets o = plan_offsets(counts, U, heavy_threshold, stats);
+    std::vector<int64_t> hs = read_stats(stats);
+    TORCH_CHECK(hs[TXS_STAT_OUT_OF_RANGE] == 0, "unq_inv holds ids outside [0, num_unq=", U, ")");
+    Tensor seg = empty_i32(N, unq_inv);
+    OptTensor perm;
+    if (hs[TXS_STAT_UNSORTED]) {
+        Tensor p = empty_i32(N, unq_inv);
+        Tensor ws = empty_i32(txs_sort_workspace_len(N, U), unq_inv);
+        check_status(txs_plan_sort(i32p(unq_inv), N, U, i32p(o.slot_of), i32w(p), i32w(seg),
+                                   i32w(ws), st),
+                     "plan_sort");
+        perm = p;
+    } else {
+        check_status(txs_plan_seg_sorted(i32p(unq_inv), N, U, i32p(o.slot_of), i32w(seg), st),
+                     "plan_seg_sorted");
+    }
+    Tensor heavy_ids = o.heavy_ids.narrow(0, 0, hs[TXS_STAT_NUM_SPECIAL]).contiguous();
+    return {o.preSum, perm, seg, o.slot_of, heavy_ids, hs};
+}
+
+// Plan for callers that hold only CSR offsets of already grouped rows.
+// returns (seg, slot_of, heavy_ids, stats)
+std::tuple<Tensor, Tensor, Tensor, std::vector<int64_t>> plan_from_presum(
+    const Tensor &preSum, int64_t num_total, int64_t heavy_threshold) {
+    check_i32(preSum, "preSum");
+    TORCH_CHECK(preSum.dim() == 1 && preSum.numel() >= 1, "preSum must be 1-D with num_unq+1 entries");
+    c10::hip::HIPGuard guard(preSum.device());
+    const int64_t U = preSum.numel() - 1, N = num_total;
+    void *st = cur_stream(preSum);
+    Tensor counts = empty_i32(U, preSum);
+    Tensor stats = empty_i32(TXS_STATS_LEN, preSum);
+    check_status(txs_counts_from_presum(i32p(preSum), U, i32w(counts), i32w(stats), st),
+                 "counts_from_presum");
+    Offsets o = plan_offsets(counts, U, heavy_threshold, stats);
+    std::vector<int64_t> hs = read_stats(stats);
+    Tensor seg = empty_i32(N, preSum);
+    check_status(txs_plan_seg_from_presum(i32p(preSum), N, U, i32p(o.slot_of), i32w(seg), st),
+                 "plan_seg_from_presum");
+    Tensor heavy_ids = o.heavy_ids.narrow(0, 0, hs[TXS_STAT_NUM_SPECIAL]).contiguous();
+    return {seg, o.slot_of, heavy_ids, hs};
+}
+
+Tensor make_scratch(int64_t num_special, int64_t C, const Tensor &like) {
+    return at::zeros({num_special * C}, like.options().dtype(at::kLong));
+}
+
+void run_forward(int op, const Tensor &feats, const OptTensor &perm, const Tensor &seg,
+                 const Tensor &preSum, const Tensor &slot_of, const Tensor &heavy_ids,
+                 Tensor &scratch, Tensor &out, OptTensor &arg) {
+    const int64_t N = feats.size(0), C = feats.size(1), U = preSum.numel() - 1;
+    const int64_t S = heavy_ids.numel();
+    TORCH_CHECK(seg.numel() == N, "plan was built for ", seg.numel(), " rows, feats has ", N);
+    TORCH_CHECK(!perm.has_value() || perm->numel() == N, "perm length mismatch");
+    TORCH_CHECK(slot_of.numel() == U, "slot_of length mismatch");
+    TORCH_CHECK(out.size(0) == U && out.size(1) == C, "out must be [num_unq, channel]");
+    TORCH_CHECK(S == 0 || scratch.numel() >= S * C, "scratch too small");
+    const int dt = dtype_code(feats, "feats");
+    void *st = cur_stream(feats);
+    int rc;
+    {
+        pybind11::gil_scoped_release nogil;
+        rc = txs_scatter_forward(op, dt, feats.data_ptr(), opt_i32p(perm), i32p(seg), i32p(preSum),
+                                 i32p(slot_of), i32p(heavy_ids), S,
+                                 S ? scratch.data_ptr() : nullptr, out.data_ptr(),
+                                 arg.has_value() ? arg->data_ptr<int32_t>() : nullptr, N, C, U, st);
+    }
+    check_status(rc, "scatter_forward");
+}
+
+// forward(op, feats, perm|None, seg, preSum, slot_of, heavy_ids, scratch) -> (out, arg|None)
+std::tuple<Tensor, OptTensor> forward(int64_t op, const Tensor &feats, const OptTensor &perm,
+                                      const Tensor &seg, const Tensor &preSum,
+                                      const Tensor &slot_of, const Tensor &heavy_ids,
+                                      Tensor scratch) {
+    check_dev(feats, "feats");
+    TORCH_CHECK(feats.dim() == 2, "feats must be [num_total, channel]");
+    check_i32(seg, "seg");
+    check_i32(preSum, "preSum");
+    check_i32(slot_of, "slot_of");
+    check_i32(heavy_ids, "heavy_ids");
+    if (perm.has_value()) check_i32(*perm, "perm");
+    check_dev(scratch, "scratch");
+    TORCH_CHECK(scratch.scalar_type() == at::kLong, "scratch must be int64");
+    TORCH_CHECK(seg.device() == feats.device(), "plan and feats live on different devices");
+    c10::hip::HIPGuard guard(feats.device());
+    const int64_t C = feats.size(1), U = preSum.numel() - 1;
+    Tensor out = at::empty({U, C}, feats.options());
+    OptTensor arg;
+    if (op == TXS_MAX) arg = at::empty({U, C}, feats.options().dtype(at::kInt));
+    run_forward((int)op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, out, arg);
+    return {out, arg};
+}
+
+// backward(op, grad_out, arg|None, perm|None, seg, preSum, num_total) -> grad_in
+Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const OptTensor &perm,
+                const Tensor &seg, const Tensor &preSum, int64_t num_total) {
+    check_dev(grad_out, "grad_out");
+    TORCH_CHECK(grad_out.dim() == 2, "grad_out must be [num_unq, channel]");
+    check_i32(seg, "seg");
+    check_i32(preSum, "preSum");
+    if (perm.has_value()) check_i32(*perm, "perm");
+    const int64_t U = preSum.numel() - 1, C = grad_out.size(1), N = num_total;
+    TORCH_CHECK(grad_out.size(0) == U, "grad_out has ", grad_out.size(0), " rows, plan has ", U, " voxels");
+    TORCH_CHECK(seg.numel() == N, "plan row count mismatch");
+    TORCH_CHECK(!perm.has_value() || perm->numel() == N, "perm length mismatch");
+    if (op == TXS_MAX) {
+        TORCH_CHECK(arg.has_value(), "scatter_max backward needs arg");
+        check_i32(*arg, "arg");
+        TORCH_CHECK(arg->dim() == 2 && arg->size(0) == U && arg->size(1) == C, "arg must be [num_unq, channel]");
+    }
+    c10::hip::HIPGuard guard(grad_out.device());
+    const int dt = dtype_code(grad_out, "grad_out");
+    Tensor gin = at::empty({N, C}, grad_out.options());
+    void *st = cur_stream(grad_out);
+    int rc;
+    {
+        pybind11::gil_scoped_release nogil;
+        rc = txs_scatter_backward((int)op, dt, grad_out.data_ptr(), opt_i32p(arg), opt_i32p(perm),
+                                  i32p(seg), i32p(preSum), gin.data_ptr(), N, C, U, st);
+    }
+    check_status(rc, "scatter_backward");
+    return gin;
+}
+
+// ---- the reference module's three functions (scatter.cpp:20-64) ------------
+
+void csr_reduce(int op, Tensor feats, Tensor preSum, Tensor out, OptTensor arg) {  // arg by value
+    check_dev(feats, "feats");
+    check_i32(preSum, "preSum");
+    check_dev(out, "out");
+    TORCH_CHECK(feats.dim() == 2 && out.dim() == 2, "feats and out must be 2-D");
+    TORCH_CHECK(out.scalar_type() == feats.scalar_type(), "out dtype must match feats");
+    TORCH_CHECK(preSum.numel() == out.size(0) + 1, "preSum must have out.size(0)+1 entries");
+    c10::hip::HIPGuard guard(feats.device());
+    auto [seg, slot_of, heavy_ids, hs] =
+        plan_from_presum(preSum, feats.size(0), txs_default_heavy_threshold());
+    Tensor scratch = make_scratch(heavy_ids.numel(), feats.size(1), feats);
+    OptTensor perm;
+    run_forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, out, arg);
+}
+
+// sum(feats, preSum, out, max_cnt): max_cnt only shaped the reference's thread
+// blocks (scatter_kernel.cu:179); it is accepted and not needed here.
+void sum_ref(Tensor feats, Tensor preSum, Tensor out, int64_t /*max_cnt*/) {
+    csr_reduce(TXS_SUM, feats, preSum, out, std::nullopt);
+}
+
+void max_ref(Tensor feats, Tensor preSum, Tensor out, Tensor arg, int64_t /*max_cnt*/) {
+    check_i32(arg, "arg");
+    TORCH_CHECK(arg.sizes() == out.sizes(), "arg must have the shape of out");
+    csr_reduce(TXS_MAX, feats, preSum, out, arg);
+}
+
+void get_presum_ref(Tensor unq_inv, Tensor preSum) {
+    check_i32(unq_inv, "unq_inv");
+    check_i32(preSum, "preSum");
+    c10::hip::HIPGuard guard(unq_inv.device());
+    check_status(txs_get_presum(i32p(unq_inv), i32w(preSum), unq_inv.numel(), preSum.numel(),
+                                cur_stream(unq_inv)),
+                 "getPreSum");
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    m.def("sum", &sum_ref, "scatter_sum over CSR offsets, in place (HIP)");
+    m.def("max", &max_ref, "scatter_max with arg over CSR offsets, in place (HIP)");
+    m.def("getPreSum", &get_presum_ref, "CSR offsets from a sorted unq_inv (HIP)");
+    m.def("build_plan", &build_plan, "index preparation for unq_inv in any order");
+    m.def("plan_from_presum", &plan_from_presum, "index preparation from CSR offsets");
+    m.def("make_scratch", &make_scratch, "zeroed scratch table for the special voxels");
+    m.def("forward", &forward, "forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch)");
+    m.def("backward", &backward, "backward(op, grad_out, arg, perm, seg, preSum, num_total)");
+    m.def("abi_version", &txs_abi_version);
+    m.def("default_heavy_threshold", &txs_default_heavy_threshold);
+    m.attr("SUM") = (int)TXS_SUM;
+    m.attr("MEAN") = (int)TXS_MEAN;
+    m.attr("MAX") = (int)TXS_MAX;
+}

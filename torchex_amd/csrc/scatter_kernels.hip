@@ -1,0 +1,979 @@
+// Voxel scatter-reduction kernels for MI355X (gfx950, wave64) and their C ABI.
+//
+// Design in one paragraph.  Index preparation sorts row ids by voxel id once
+// (stable LSD radix sort) and stores, for every sorted position j, the row
+// perm[j] and the voxel seg[j].  The forward pass is then a segmented reduction
+// over sorted positions: a "lane group" (the lanes that together cover one
+// feature row, each lane owning one 128-bit channel vector) walks a fixed-size
+// chunk of positions, keeps the running sum / max of the current voxel in
+// registers and writes a voxel's output row exactly once when its run of equal
+// ids ends.  A run that starts in a chunk is finished by the same lane group
+// even if it spills into the next chunk, so ordinary voxels never need an
+// atomic.  Only voxels above the heavy threshold are split across lane groups;
+// their per-chunk partials meet in a scratch table through fp32 atomic adds
+// (sum/mean) or a 64-bit atomic max on a packed (ordered value | ~row) word
+// (max/argmax), and a small finalize kernel turns the table into output rows.
+// The backward pass is a gather over the same sorted positions: the upstream
+// row of a voxel is read once per position from cache and every row of the
+// input gradient is written exactly once, with no zero-fill pass and no atomics.
+//
+// Reference behaviour being replaced: torchex/src/scatter/scatter_kernel.cu
+// (getPreSum :85-100, scatter_sum :102-129, scatter_max :131-171) and the
+// tensor arithmetic of torchex/operator_py/scatter_op.py (:47-50, :69, :74-78,
+// :106-111).
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "torchex_scatter.h"
+
+namespace {
+
+constexpr int kThreads = 256;        // 4 wavefronts per workgroup
+constexpr int kChunk = 32;           // sorted positions per lane group
+constexpr int kBatch = 8;            // rows in flight per lane group
+constexpr int kHeavyDefault = 64;    // voxels above this many rows use the atomic path
+constexpr int kSpecialBit = (int)0x80000000;
+constexpr int kIdMask = 0x7fffffff;
+
+// ------------------------------------------------------------------ dtypes --
+
+struct F32 {
+    using raw = float;
+    static __device__ __forceinline__ float to_f(raw x) { return x; }
+    static __device__ __forceinline__ raw from_f(float x) { return x; }
+    static __device__ __forceinline__ raw lowest() { return -3.402823466e+38f; }
+    static __device__ __forceinline__ raw zero() { return 0.0f; }
+};
+struct F16 {
+    using raw = _Float16;
+    static __device__ __forceinline__ float to_f(raw x) { return (float)x; }
+    static __device__ __forceinline__ raw from_f(float x) { return (_Float16)x; }  // RNE
+    static __device__ __forceinline__ raw lowest() { return (_Float16)(-65504.0f); }
+    static __device__ __forceinline__ raw zero() { return (_Float16)0.0f; }
+};
+struct BF16 {
+    using raw = unsigned short;
+    static __device__ __forceinline__ float to_f(raw x) {
+        return __uint_as_float(((unsigned)x) << 16);
+    }
+    static __device__ __forceinline__ raw from_f(float x) {  // round to nearest even
+        unsigned b = __float_as_uint(x);
+        if ((b & 0x7fffffffu) > 0x7f800000u) return (raw)((b >> 16) | 0x0040u);
+        b += 0x7fffu + ((b >> 16) & 1u);
+        return (raw)(b >> 16);
+    }
+    static __device__ __forceinline__ raw lowest() { return (raw)0xff7f; }
+    static __device__ __forceinline__ raw zero() { return (raw)0; }
+};
+
+// VEC consecutive elements moved by one lane with a single memory instruction.
+template <typename T, int VEC>
+struct alignas(sizeof(T) * VEC) Pack {
+    T v[VEC];
+};
+
+template <typename T, int VEC>
+__device__ __forceinline__ Pack<T, VEC> ld(const T *p) {
+    return *reinterpret_cast<const Pack<T, VEC> *>(p);
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void st(T *p, const Pack<T, VEC> &x) {
+    *reinterpret_cast<Pack<T, VEC> *>(p) = x;
+}
+
+// Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous
+// range of chunks so neighbouring chunks (which share voxels, seg/perm cache
+// lines and upstream-gradient rows) meet in the same L2.  gridDim.x is a
+// multiple of 8.
+__device__ __forceinline__ int xcd_block(int b, int nb) { return (b & 7) * (nb >> 3) + (b >> 3); }
+
+// Monotonic map from non-NaN floats to unsigned ints; -0.0 is folded into +0.0
+// first so the two zeros tie, as they do under the reference's float compare.
+__device__ __forceinline__ unsigned ordered_bits(float v) {
+    unsigned b = __float_as_uint(v + 0.0f);
+    return b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u);
+}
+
+// -------------------------------------------------------------- small utils --
+
+__global__ void fill_i32_kernel(int *p, long n, int value) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = value;
+}
+
+// Reference getPreSum (scatter_kernel.cu:85-100) for sorted ids.
+__global__ void get_presum_kernel(const int *__restrict__ inv, int *__restrict__ preSum, long n,
+                                  long num_presum) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    int v = inv[i];
+    bool boundary = (i == n - 1) || (inv[i + 1] != v);
+    long slot = (long)v + 1;
+    if (boundary && slot >= 0 && slot < num_presum) preSum[slot] = (int)(i + 1);
+}
+
+__global__ void plan_count_kernel(const int *__restrict__ inv, long n, int U,
+                                  int *__restrict__ counts, int *__restrict__ stats) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    int v = inv[i];
+    if ((unsigned)v >= (unsigned)U) {
+        stats[TXS_STAT_OUT_OF_RANGE] = 1;
+        return;
+    }
+    atomicAdd(&counts[v], 1);
+    if (i + 1 < n && inv[i + 1] < v) stats[TXS_STAT_UNSORTED] = 1;
+}
+
+__global__ void counts_from_presum_kernel(const int *__restrict__ preSum, int U,
+                                          int *__restrict__ counts) {
+    int u = blockIdx.x * blockDim.x + threadIdx.x;
+    if (u < U) counts[u] = preSum[u + 1] - preSum[u];
+}
+
+// ------------------------------------------------------------ exclusive scan --
+// out[i] = sum_{k<i} in[k] for i in [0, n_out), where in[k] = 0 for k >= n_in.
+// Three launches, no inter-block waiting: tile sums, scan of tile sums by one
+// workgroup, tile-local scan plus tile offset.
+
+constexpr int kScanItems = 8;
+constexpr int kScanTile = kThreads * kScanItems;
+
+__device__ __forceinline__ int wave_inclusive_scan(int x) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        int y = __shfl_up(x, d, 64);
+        if (lane >= d) x += y;
+    }
+    return x;
+}
+
+// exclusive scan of one int per thread across the 256-thread workgroup;
+// *total receives the workgroup sum
+__device__ __forceinline__ int block_exclusive_scan(int x, int *total) {
+    __shared__ int wsum[kThreads / 64];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    int inc = wave_inclusive_scan(x);
+    __syncthreads();  // wsum may still be read by a previous call
+    if (lane == 63) wsum[w] = inc;
+    __syncthreads();
+    int off = 0, tot = 0;
+#pragma unroll
+    for (int k = 0; k < kThreads / 64; ++k) {
+        int s = wsum[k];
+        if (k < w) off += s;
+        tot += s;
+    }
+    *total = tot;
+    return off + inc - x;
+}
+
+__global__ __launch_bounds__(kThreads) void scan_tile_sums_kernel(const int *__restrict__ in,
+                                                                  long n_in,
+                                                                  int *__restrict__ tile_sums) {
+    long base = (long)blockIdx.x * kScanTile + (long)threadIdx.x * kScanItems;
+    int s = 0;
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+        long i = base + k;
+        if (i < n_in) s += in[i];
+    }
+    int tot;
+    block_exclusive_scan(s, &tot);
+    if (threadIdx.x == 0) tile_sums[blockIdx.x] = tot;
+}
+
+__global__ __launch_bounds__(kThreads) void scan_tile_offsets_kernel(int *__restrict__ tile_sums,
+                                                                     long n_tiles) {
+    int carry = 0;
+    for (long base = 0; base < n_tiles; base += kThreads) {
+        long i = base + threadIdx.x;
+        int x = (i < n_tiles) ? tile_sums[i] : 0;
+        int tot;
+        int ex = block_exclusive_scan(x, &tot);
+        if (i < n_tiles) tile_sums[i] = carry + ex;
+        carry += tot;
+    }
+}
+
+// in and out may be the same array: a thread reads its items before any write
+__global__ __launch_bounds__(kThreads) void scan_apply_kernel(const int *in, long n_in, int *out,
+                                                              long n_out, const int *tile_offs) {
+    long base = (long)blockIdx.x * kScanTile + (long)threadIdx.x * kScanItems;
+    int x[kScanItems];
+    int s = 0;
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+        long i = base + k;
+        x[k] = (i < n_in) ? in[i] : 0;
+        s += x[k];
+    }
+    int tot;
+    int run = block_exclusive_scan(s, &tot) + tile_offs[blockIdx.x];
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+        long i = base + k;
+        if (i < n_out) out[i] = run;
+        run += x[k];
+    }
+}
+
+long scan_tiles(long n_out) { return (n_out + kScanTile - 1) / kScanTile; }
+
+hipError_t exclusive_scan(const int *in, long n_in, int *out, long n_out, int *ws,
+                          hipStream_t st) {
+    if (n_out <= 0) return hipSuccess;
+    long tiles = scan_tiles(n_out);
+    scan_tile_sums_kernel<<<dim3((unsigned)tiles), dim3(kThreads), 0, st>>>(in, n_in, ws);
+    scan_tile_offsets_kernel<<<dim3(1), dim3(kThreads), 0, st>>>(ws, tiles);
+    scan_apply_kernel<<<dim3((unsigned)tiles), dim3(kThreads), 0, st>>>(in, n_in, out, n_out, ws);
+    return hipGetLastError();
+}
+
+// special-voxel table and max_cnt
+__global__ void plan_special_kernel(const int *__restrict__ counts, int U, int heavy_threshold,
+                                    int *__restrict__ slot_of, int *__restrict__ heavy_ids,
+                                    int *__restrict__ stats) {
+    int u = blockIdx.x * blockDim.x + threadIdx.x;
+    if (u >= U) return;
+    int c = counts[u];
+    atomicMax(&stats[TXS_STAT_MAX_CNT], c);
+    int slot = -1;
+    if (c == 0) atomicAdd(&stats[TXS_STAT_NUM_EMPTY], 1);
+    if (c > heavy_threshold || c == 0) {
+        slot = atomicAdd(&stats[TXS_STAT_NUM_SPECIAL], 1);
+        if (slot < U) heavy_ids[slot] = u;
+    }
+    slot_of[u] = slot;
+}
+
+// ----------------------------------------------------------- stable radix sort --
+// One pass = per-tile digit histogram, exclusive scan of the digit-major
+// histogram, stable scatter.  Inside a tile the order is (wave, item, lane),
+// i.e. ascending input index, so each pass is stable.
+
+constexpr int kSortItems = 8;
+constexpr int kSortTile = kThreads * kSortItems;  // 2048 keys per workgroup
+constexpr int kSortWaves = kThreads / 64;
+constexpr int kSortWaveSpan = 64 * kSortItems;    // 512 consecutive keys per wave
+
+__global__ __launch_bounds__(kThreads) void sort_hist_kernel(const int *__restrict__ keys, long n,
+                                                             int shift, int rbits,
+                                                             int *__restrict__ hist, int n_tiles) {
+    __shared__ int h[256];
+    const int R = 1 << rbits;
+    h[threadIdx.x] = 0;
+    __syncthreads();
+    long base = (long)blockIdx.x * kSortTile;
+#pragma unroll
+    for (int it = 0; it < kSortItems; ++it) {
+        long i = base + (long)it * kThreads + threadIdx.x;
+        if (i < n) atomicAdd(&h[(keys[i] >> shift) & (R - 1)], 1);
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < R) hist[(long)threadIdx.x * n_tiles + blockIdx.x] = h[threadIdx.x];
+}
+
+__global__ __launch_bounds__(kThreads) void sort_scatter_kernel(
+    const int *__restrict__ keys_in, const int *__restrict__ vals_in, int *__restrict__ keys_out,
+    int *__restrict__ vals_out, long n, int shift, int rbits, const int *__restrict__ hist_scanned,
+    int n_tiles) {
+    __shared__ int wcount[kSortWaves][256];
+    __shared__ int woff[kSortWaves][256];
+    const int R = 1 << rbits;
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const unsigned long long lanes_below = (1ull << lane) - 1ull;
+    for (int k = threadIdx.x; k < kSortWaves * 256; k += kThreads) (&wcount[0][0])[k] = 0;
+    __syncthreads();
+
+    const long base = (long)blockIdx.x * kSortTile + (long)w * kSortWaveSpan;
+    int key[kSortItems], lrank[kSortItems];
+    volatile int *wc = &wcount[w][0];
+#pragma unroll
+    for (int it = 0; it < kSortItems; ++it) {
+        long i = base + (long)it * 64 + lane;
+        bool valid = i < n;
+        key[it] = valid ? keys_in[i] : 0;
+        int digit = (key[it] >> shift) & (R - 1);
+        unsigned long long mask = __ballot(valid);
+        for (int b = 0; b < rbits; ++b) {
+            bool bit = (digit >> b) & 1;
+            unsigned long long bal = __ballot(bit);
+            mask &= bit ? bal : ~bal;
+        }
+        int below = __popcll(mask & lanes_below);
+        int prev = wc[digit];
+        __builtin_amdgcn_wave_barrier();
+        if (valid && below == 0) wc[digit] = prev + __popcll(mask);
+        __builtin_amdgcn_wave_barrier();
+        lrank[it] = prev + below;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < R) {
+        int run = hist_scanned[(long)threadIdx.x * n_tiles + blockIdx.x];
+#pragma unroll
+        for (int k = 0; k < kSortWaves; ++k) {
+            woff[k][threadIdx.x] = run;
+            run += wcount[k][threadIdx.x];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < kSortItems; ++it) {
+        long i = base + (long)it * 64 + lane;
+        if (i < n) {
+            int digit = (key[it] >> shift) & (R - 1);
+            long dst = (long)woff[w][digit] + lrank[it];
+            if (dst >= 0 && dst < n) {
+                keys_out[dst] = key[it];
+                vals_out[dst] = vals_in ? vals_in[i] : (int)i;
+            }
+        }
+    }
+}
+
+// seg[j] = id | special bit
+__global__ void seg_flag_kernel(const int *__restrict__ ids, long n, int U,
+                                const int *__restrict__ slot_of, int *__restrict__ seg) {
+    long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    int u = ids[j] & kIdMask;
+    int flag = ((unsigned)u < (unsigned)U && slot_of[u] >= 0) ? kSpecialBit : 0;
+    seg[j] = u | flag;
+}
+
+// seg by binary search of each position in preSum (largest u with preSum[u] <= j)
+__global__ void seg_from_presum_kernel(const int *__restrict__ preSum, long n, int U,
+                                       const int *__restrict__ slot_of, int *__restrict__ seg) {
+    long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    int lo = 0, hi = U;  // invariant: preSum[lo] <= j < preSum[hi]
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if ((long)preSum[mid] <= j) lo = mid; else hi = mid;
+    }
+    int flag = (slot_of[lo] >= 0) ? kSpecialBit : 0;
+    seg[j] = lo | flag;
+}
+
+// ----------------------------------------------------------------- forward --
+
+template <class TR, int VEC, int OP>
+__global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
+    const typename TR::raw *__restrict__ feats, const int *__restrict__ perm,
+    const int *__restrict__ seg, const int *__restrict__ preSum, const int *__restrict__ slot_of,
+    typename TR::raw *__restrict__ out, int *__restrict__ arg,
+    unsigned long long *__restrict__ scratch, int N, int C, int U, int lpr_log2, int n_groups) {
+    using raw = typename TR::raw;
+    const int group = xcd_block(blockIdx.x, gridDim.x) * (kThreads >> lpr_log2) +
+                      ((int)threadIdx.x >> lpr_log2);
+    const int col = ((int)blockIdx.y << lpr_log2 | ((int)threadIdx.x & ((1 << lpr_log2) - 1))) * VEC;
+    if (group >= n_groups || col >= C) return;
+
+    // Range of sorted positions [a, b) this lane group reduces: its chunk,
+    // minus the tail of an ordinary run that began in an earlier chunk, plus
+    // the tail of an ordinary run that begins here and ends later.
+    int a = group * kChunk;
+    const int chunk_end = min(N, a + kChunk);
+    {
+        int s0 = seg[a];
+        if (a > 0 && s0 >= 0 && seg[a - 1] == s0) a = preSum[s0 + 1];
+    }
+    if (a >= chunk_end) return;
+    int b = chunk_end;
+    if (chunk_end < N) {
+        int sl = seg[chunk_end - 1];
+        if (sl >= 0 && seg[chunk_end] == sl) b = min(N, preSum[sl + 1]);
+    }
+
+    float acc[VEC];
+    int idx[VEC];
+    int cur = seg[a];
+    int run_j0 = a;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        acc[k] = (OP == TXS_MAX) ? -__builtin_inff() : 0.0f;
+        idx[k] = -1;
+    }
+
+    // Emit the finished run [run_j0, run_end) of voxel `cur`.
+    auto flush = [&](int run_end) {
+        const int u = cur & kIdMask;
+        if ((unsigned)u >= (unsigned)U) return;
+        if (OP == TXS_MAX) {
+            bool missing = false;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) missing |= idx[k] < 0;
+            if (__builtin_expect(missing, 0)) {
+                // No value above -inf was seen in some channel: the run holds
+                // only -inf and NaN there.  The first -inf row wins.
+                for (int p = run_j0; p < run_end; ++p) {
+                    int row = perm ? perm[p] : p;
+                    if ((unsigned)row >= (unsigned)N) continue;
+                    Pack<raw, VEC> x = ld<raw, VEC>(feats + (size_t)row * C + col);
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k)
+                        if (idx[k] < 0 && TR::to_f(x.v[k]) == -__builtin_inff()) idx[k] = row;
+                }
+            }
+        }
+        if (cur >= 0) {  // ordinary voxel: the whole run was reduced here
+            const size_t o = (size_t)u * C + col;
+            Pack<raw, VEC> r;
+            if (OP == TXS_SUM) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) r.v[k] = TR::from_f(acc[k]);
+            } else if (OP == TXS_MEAN) {
+                const float d = (float)(run_end - run_j0);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) r.v[k] = TR::from_f(acc[k] / d);
+            } else {
+                Pack<int, VEC> ai;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    r.v[k] = idx[k] >= 0 ? TR::from_f(acc[k]) : TR::lowest();
+                    ai.v[k] = idx[k];
+                }
+                st<int, VEC>(arg + o, ai);
+            }
+            st<raw, VEC>(out + o, r);
+        } else {  // heavy voxel: merge this chunk's partial into the scratch table
+            const int slot = slot_of[u];
+            if (slot < 0) return;
+            const size_t o = (size_t)slot * C + col;
+            if (OP == TXS_MAX) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    if (idx[k] >= 0) {
+                        unsigned long long key = ((unsigned long long)ordered_bits(acc[k]) << 32) |
+                                                 (unsigned long long)(0xffffffffu - (unsigned)idx[k]);
+                        atomicMax(scratch + o + k, key);
+                    }
+                }
+            } else {
+                float *fs = reinterpret_cast<float *>(scratch) + o;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) unsafeAtomicAdd(fs + k, acc[k]);
+            }
+        }
+    };
+
+    for (int j = a; j < b; j += kBatch) {
+        int segs[kBatch], rows[kBatch];
+        Pack<raw, VEC> v[kBatch];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const int jj = j + i;
+            const bool ok = jj < b;
+            const int js = ok ? jj : a;
+            segs[i] = seg[js];
+            int r = perm ? perm[js] : js;
+            rows[i] = (ok && (unsigned)r < (unsigned)N) ? r : -1;
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i)
+            if (rows[i] >= 0) v[i] = ld<raw, VEC>(feats + (size_t)rows[i] * C + col);
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            if (rows[i] < 0) continue;
+            if (segs[i] != cur) {
+                flush(j + i);
+                cur = segs[i];
+                run_j0 = j + i;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    acc[k] = (OP == TXS_MAX) ? -__builtin_inff() : 0.0f;
+                    idx[k] = -1;
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                const float x = TR::to_f(v[i].v[k]);
+                if (OP == TXS_MAX) {
+                    const bool take = x > acc[k];  // strict: first row wins ties, NaN never wins
+                    acc[k] = take ? x : acc[k];
+                    idx[k] = take ? rows[i] : idx[k];
+                } else {
+                    acc[k] += x;
+                }
+            }
+        }
+    }
+    flush(b);
+}
+
+// Turn the scratch table of the special voxels into output rows and clear it.
+template <class TR, int OP>
+__global__ void scatter_finalize_kernel(const typename TR::raw *__restrict__ feats,
+                                        const int *__restrict__ preSum,
+                                        const int *__restrict__ heavy_ids,
+                                        unsigned long long *__restrict__ scratch,
+                                        typename TR::raw *__restrict__ out,
+                                        int *__restrict__ arg, int n_special, int N, int C, int U) {
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= (long)n_special * C) return;
+    const int s = (int)(t / C), c = (int)(t - (long)s * C);
+    const int u = heavy_ids[s];
+    if ((unsigned)u >= (unsigned)U) return;
+    const size_t o = (size_t)u * C + c;
+    if (OP == TXS_MAX) {
+        const unsigned long long key = scratch[t];
+        scratch[t] = 0ull;
+        const unsigned row = 0xffffffffu - (unsigned)(key & 0xffffffffull);
+        if (key == 0ull || row >= (unsigned)N) {
+            out[o] = TR::lowest();
+            arg[o] = -1;
+        } else {
+            out[o] = feats[(size_t)row * C + c];  // exact bits of the winner
+            arg[o] = (int)row;
+        }
+    } else {
+        float *fs = reinterpret_cast<float *>(scratch);
+        float s32 = fs[t];
+        fs[t] = 0.0f;
+        if (OP == TXS_MEAN) s32 = s32 / (float)(preSum[u + 1] - preSum[u]);
+        out[o] = TR::from_f(s32);
+    }
+}
+
+// ---------------------------------------------------------------- backward --
+
+template <class TR, int VEC, int OP>
+__global__ __launch_bounds__(kThreads) void scatter_bwd_kernel(
+    const typename TR::raw *__restrict__ g, const int *__restrict__ arg,
+    const int *__restrict__ perm, const int *__restrict__ seg, const int *__restrict__ preSum,
+    typename TR::raw *__restrict__ gin, int N, int C, int U, int lpr_log2, int n_groups) {
+    using raw = typename TR::raw;
+    const int group = xcd_block(blockIdx.x, gridDim.x) * (kThreads >> lpr_log2) +
+                      ((int)threadIdx.x >> lpr_log2);
+    const int col = ((int)blockIdx.y << lpr_log2 | ((int)threadIdx.x & ((1 << lpr_log2) - 1))) * VEC;
+    if (group >= n_groups || col >= C) return;
+    const int a = group * kChunk;
+    const int b = min(N, a + kChunk);
+
+    int cur = -1;  // voxel whose scaled gradient row is held in q (mean only)
+    Pack<raw, VEC> q;
+    for (int j = a; j < b; j += kBatch) {
+        int us[kBatch], rows[kBatch];
+        Pack<raw, VEC> gv[kBatch];
+        Pack<int, VEC> av[kBatch];
+        int c0[kBatch], c1[kBatch];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const int jj = j + i;
+            const bool ok = jj < b;
+            const int js = ok ? jj : a;
+            const int u = seg[js] & kIdMask;
+            const int r = perm ? perm[js] : js;
+            us[i] = u;
+            rows[i] = (ok && (unsigned)r < (unsigned)N && (unsigned)u < (unsigned)U) ? r : -1;
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            if (rows[i] < 0) continue;
+            const size_t o = (size_t)us[i] * C + col;
+            gv[i] = ld<raw, VEC>(g + o);
+            if (OP == TXS_MAX) av[i] = ld<int, VEC>(arg + o);
+            if (OP == TXS_MEAN) {
+                c0[i] = preSum[us[i]];
+                c1[i] = preSum[us[i] + 1];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            if (rows[i] < 0) continue;
+            Pack<raw, VEC> r;
+            if (OP == TXS_SUM) {
+                r = gv[i];
+            } else if (OP == TXS_MEAN) {
+                if (us[i] != cur) {  // one division per run, not per row
+                    cur = us[i];
+                    const float d = (float)(c1[i] - c0[i]);
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) q.v[k] = TR::from_f(TR::to_f(gv[i].v[k]) / d);
+                }
+                r = q;
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k)
+                    r.v[k] = (av[i].v[k] == rows[i]) ? gv[i].v[k] : TR::zero();
+            }
+            st<raw, VEC>(gin + (size_t)rows[i] * C + col, r);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ launch --
+
+struct Geometry {
+    int vec_bytes;  // bytes one lane moves per row
+    int lpr_log2;   // log2(lanes that cover one row slice)
+    int ytiles;     // column tiles when a row is wider than 64 lanes
+    int n_groups;
+    dim3 grid;
+};
+
+bool aligned_to(const void *p, int bytes) { return p == nullptr || ((uintptr_t)p % (uintptr_t)bytes) == 0; }
+
+Geometry make_geometry(long N, long C, int elem, const void *p0, const void *p1, const void *p2,
+                       bool arg_used, const void *parg) {
+    Geometry g;
+    int vb = 16;
+    while (vb > elem) {
+        int vec = vb / elem;
+        bool ok = (C * elem) % vb == 0 && aligned_to(p0, vb) && aligned_to(p1, vb) && aligned_to(p2, vb);
+        if (arg_used) ok = ok && aligned_to(parg, vec * 4);
+        if (ok) break;
+        vb >>= 1;
+    }
+    g.vec_bytes = vb;
+    const long vec = vb / elem;
+    const long lanes = (C + vec - 1) / vec;
+    int l2 = 0;
+    while ((1L << l2) < lanes && l2 < 6) ++l2;
+    g.lpr_log2 = l2;
+    g.ytiles = (int)((lanes + (1L << l2) - 1) >> l2);
+    g.n_groups = (int)((N + kChunk - 1) / kChunk);
+    const long groups_per_block = kThreads >> l2;
+    long blocks = (g.n_groups + groups_per_block - 1) / groups_per_block;
+    blocks = (blocks + 7) & ~7L;
+    g.grid = dim3((unsigned)blocks, (unsigned)g.ytiles, 1);
+    return g;
+}
+
+template <class TR, int VEC>
+hipError_t launch_fwd_op(int op, const Geometry &geo, hipStream_t st, const void *feats,
+                         const int *perm, const int *seg, const int *preSum, const int *slot_of,
+                         void *out, int *arg, void *scratch, int N, int C, int U) {
+    using raw = typename TR::raw;
+    auto f = (const raw *)feats;
+    auto o = (raw *)out;
+    auto s = (unsigned long long *)scratch;
+    dim3 blk(kThreads);
+    switch (op) {
+        case TXS_SUM:
+            scatter_fwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, 0, st>>>(
+                f, perm, seg, preSum, slot_of, o, arg, s, N, C, U, geo.lpr_log2, geo.n_groups);
+            break;
+        case TXS_MEAN:
+            scatter_fwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, 0, st>>>(
+                f, perm, seg, preSum, slot_of, o, arg, s, N, C, U, geo.lpr_log2, geo.n_groups);
+            break;
+        default:
+            scatter_fwd_kernel<TR, VEC, TXS_MAX><<<geo.grid, blk, 0, st>>>(
+                f, perm, seg, preSum, slot_of, o, arg, s, N, C, U, geo.lpr_log2, geo.n_groups);
+            break;
+    }
+    return hipGetLastError();
+}
+
+template <class TR>
+hipError_t launch_fwd(int op, const Geometry &geo, hipStream_t st, const void *feats,
+                      const int *perm, const int *seg, const int *preSum, const int *slot_of,
+                      void *out, int *arg, void *scratch, int N, int C, int U) {
+    constexpr int e = (int)sizeof(typename TR::raw);
+#define TXS_FWD(VB)                                                                              \
+    if (geo.vec_bytes == VB)                                                                     \
+        return launch_fwd_op<TR, (VB) / e>(op, geo, st, feats, perm, seg, preSum, slot_of, out,  \
+                                           arg, scratch, N, C, U);
+    TXS_FWD(16)
+    TXS_FWD(8)
+    TXS_FWD(4)
+    if constexpr (e == 2) {
+        TXS_FWD(2)
+    }
+#undef TXS_FWD
+    return hipErrorInvalidValue;
+}
+
+template <class TR>
+hipError_t launch_finalize(int op, hipStream_t st, const void *feats, const int *preSum,
+                           const int *heavy_ids, void *scratch, void *out, int *arg,
+                           long n_special, int N, int C, int U) {
+    using raw = typename TR::raw;
+    const long total = n_special * C;
+    if (total <= 0) return hipSuccess;
+    dim3 grid((unsigned)((total + kThreads - 1) / kThreads)), blk(kThreads);
+    auto f = (const raw *)feats;
+    auto o = (raw *)out;
+    auto s = (unsigned long long *)scratch;
+    switch (op) {
+        case TXS_SUM:
+            scatter_finalize_kernel<TR, TXS_SUM><<<grid, blk, 0, st>>>(f, preSum, heavy_ids, s, o, arg,
+                                                                      (int)n_special, N, C, U);
+            break;
+        case TXS_MEAN:
+            scatter_finalize_kernel<TR, TXS_MEAN><<<grid, blk, 0, st>>>(f, preSum, heavy_ids, s, o,
+                                                                       arg, (int)n_special, N, C, U);
+            break;
+        default:
+            scatter_finalize_kernel<TR, TXS_MAX><<<grid, blk, 0, st>>>(f, preSum, heavy_ids, s, o, arg,
+                                                                      (int)n_special, N, C, U);
+            break;
+    }
+    return hipGetLastError();
+}
+
+template <class TR, int VEC>
+hipError_t launch_bwd_op(int op, const Geometry &geo, hipStream_t st, const void *g, const int *arg,
+                         const int *perm, const int *seg, const int *preSum, void *gin, int N, int C,
+                         int U) {
+    using raw = typename TR::raw;
+    auto gi = (const raw *)g;
+    auto go = (raw *)gin;
+    dim3 blk(kThreads);
+    switch (op) {
+        case TXS_SUM:
+            scatter_bwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, 0, st>>>(
+                gi, arg, perm, seg, preSum, go, N, C, U, geo.lpr_log2, geo.n_groups);
+            break;
+        case TXS_MEAN:
+            scatter_bwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, 0, st>>>(
+                gi, arg, perm, seg, preSum, go, N, C, U, geo.lpr_log2, geo.n_groups);
+            break;
+        default:
+            scatter_bwd_kernel<TR, VEC, TXS_MAX><<<geo.grid, blk, 0, st>>>(
+                gi, arg, perm, seg, preSum, go, N, C, U, geo.lpr_log2, geo.n_groups);
+            break;
+    }
+    return hipGetLastError();
+}
+
+template <class TR>
+hipError_t launch_bwd(int op, const Geometry &geo, hipStream_t st, const void *g, const int *arg,
+                      const int *perm, const int *seg, const int *preSum, void *gin, int N, int C,
+                      int U) {
+    constexpr int e = (int)sizeof(typename TR::raw);
+#define TXS_BWD(VB)                                                                               \
+    if (geo.vec_bytes == VB)                                                                      \
+        return launch_bwd_op<TR, (VB) / e>(op, geo, st, g, arg, perm, seg, preSum, gin, N, C, U);
+    TXS_BWD(16)
+    TXS_BWD(8)
+    TXS_BWD(4)
+    if constexpr (e == 2) {
+        TXS_BWD(2)
+    }
+#undef TXS_BWD
+    return hipErrorInvalidValue;
+}
+
+int status_of(hipError_t e) { return e == hipSuccess ? TXS_OK : TXS_ERR_LAUNCH; }
+
+// extents are int32 on the device; the margin keeps chunk arithmetic from wrapping
+bool fits_i32(int64_t x) { return x >= 0 && x < 2147483647LL - 4096; }
+
+unsigned blocks_for(long n, int per = kThreads) { return (unsigned)((n + per - 1) / per); }
+
+int radix_bits(int64_t U) {
+    int bits = 1;
+    while ((1LL << bits) < U) ++bits;
+    return bits;
+}
+
+}  // namespace
+
+// =================================================================== C ABI ==
+
+extern "C" {
+
+int txs_abi_version(void) { return 1; }
+
+const char *txs_status_string(int status) {
+    switch (status) {
+        case TXS_OK: return "ok";
+        case TXS_ERR_INVALID_ARG: return "invalid argument (null pointer, negative or oversized extent)";
+        case TXS_ERR_LAUNCH: return "HIP kernel launch failed";
+        case TXS_ERR_UNSUPPORTED: return "unsupported dtype or operator";
+        default: return "unknown status";
+    }
+}
+
+int txs_default_heavy_threshold(void) { return kHeavyDefault; }
+int txs_chunk_rows(void) { return kChunk; }
+
+int txs_get_presum(const int32_t *unq_inv, int32_t *preSum, int64_t num_total, int64_t num_presum,
+                   void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_presum)) return TXS_ERR_INVALID_ARG;
+    if (num_total == 0) return TXS_OK;
+    if (!unq_inv || !preSum) return TXS_ERR_INVALID_ARG;
+    get_presum_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+        unq_inv, preSum, num_total, num_presum);
+    return status_of(hipGetLastError());
+}
+
+int txs_plan_count(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, int32_t *counts,
+                   int32_t *stats, void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_unq) || !stats) return TXS_ERR_INVALID_ARG;
+    if ((num_total > 0 && !unq_inv) || (num_unq > 0 && !counts)) return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    fill_i32_kernel<<<dim3(1), dim3(64), 0, st>>>(stats, TXS_STATS_LEN, 0);
+    if (num_unq > 0)
+        fill_i32_kernel<<<dim3(blocks_for(num_unq)), dim3(kThreads), 0, st>>>(counts, num_unq, 0);
+    if (num_total > 0)
+        plan_count_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, st>>>(
+            unq_inv, num_total, (int)num_unq, counts, stats);
+    return status_of(hipGetLastError());
+}
+
+int64_t txs_scan_workspace_len(int64_t n) { return scan_tiles(n + 1) + 1; }
+
+int txs_plan_offsets(const int32_t *counts, int64_t num_unq, int32_t heavy_threshold,
+                     int32_t *preSum, int32_t *slot_of, int32_t *heavy_ids, int32_t *stats,
+                     int32_t *scan_ws, void *stream) {
+    if (!fits_i32(num_unq) || !preSum || !stats || !scan_ws || heavy_threshold < kChunk)
+        return TXS_ERR_INVALID_ARG;
+    if (num_unq > 0 && (!counts || !slot_of || !heavy_ids)) return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = exclusive_scan(counts, num_unq, preSum, num_unq + 1, scan_ws, st);
+    if (e != hipSuccess) return TXS_ERR_LAUNCH;
+    if (num_unq > 0)
+        plan_special_kernel<<<dim3(blocks_for(num_unq)), dim3(kThreads), 0, st>>>(
+            counts, (int)num_unq, heavy_threshold, slot_of, heavy_ids, stats);
+    return status_of(hipGetLastError());
+}
+
+int64_t txs_sort_workspace_len(int64_t num_total, int64_t num_unq) {
+    const int64_t tiles = (num_total + kSortTile - 1) / kSortTile;
+    const int64_t hist = 256 * (tiles > 0 ? tiles : 1);
+    (void)num_unq;
+    // two ping-pong arrays, the digit-major histogram, and the scan workspace
+    return 2 * num_total + hist + txs_scan_workspace_len(hist) + 16;
+}
+
+int txs_plan_sort(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
+                  const int32_t *slot_of, int32_t *perm, int32_t *seg, int32_t *sort_ws,
+                  void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_unq)) return TXS_ERR_INVALID_ARG;
+    if (num_total == 0) return TXS_OK;
+    if (!unq_inv || !slot_of || !perm || !seg || !sort_ws || num_unq <= 0) return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const long n = num_total;
+    const int n_tiles = (int)((n + kSortTile - 1) / kSortTile);
+    const long hist_len = 256L * n_tiles;
+    int *tmp_keys = sort_ws;
+    int *tmp_vals = sort_ws + n;
+    int *hist = sort_ws + 2 * n;
+    int *scan_ws = hist + hist_len;
+
+    const int bits = radix_bits(num_unq);
+    const int passes = (bits + 7) / 8;
+    const int rbits = (bits + passes - 1) / passes;
+    const int *kin = unq_inv;
+    const int *vin = nullptr;  // identity
+    for (int p = 0; p < passes; ++p) {
+        const bool to_final = ((passes - 1 - p) % 2) == 0;
+        int *kout = to_final ? seg : tmp_keys;
+        int *vout = to_final ? perm : tmp_vals;
+        const int shift = p * rbits;
+        sort_hist_kernel<<<dim3(n_tiles), dim3(kThreads), 0, st>>>(kin, n, shift, rbits, hist, n_tiles);
+        const long used = (1L << rbits) * n_tiles;
+        if (exclusive_scan(hist, used, hist, used, scan_ws, st) != hipSuccess) return TXS_ERR_LAUNCH;
+        sort_scatter_kernel<<<dim3(n_tiles), dim3(kThreads), 0, st>>>(kin, vin, kout, vout, n, shift,
+                                                                     rbits, hist, n_tiles);
+        kin = kout;
+        vin = vout;
+    }
+    seg_flag_kernel<<<dim3(blocks_for(n)), dim3(kThreads), 0, st>>>(seg, n, (int)num_unq, slot_of, seg);
+    return status_of(hipGetLastError());
+}
+
+int txs_plan_seg_sorted(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
+                        const int32_t *slot_of, int32_t *seg, void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_unq)) return TXS_ERR_INVALID_ARG;
+    if (num_total == 0) return TXS_OK;
+    if (!unq_inv || !slot_of || !seg) return TXS_ERR_INVALID_ARG;
+    seg_flag_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+        unq_inv, num_total, (int)num_unq, slot_of, seg);
+    return status_of(hipGetLastError());
+}
+
+int txs_counts_from_presum(const int32_t *preSum, int64_t num_unq, int32_t *counts, int32_t *stats,
+                           void *stream) {
+    if (!fits_i32(num_unq) || !preSum || !stats) return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    fill_i32_kernel<<<dim3(1), dim3(64), 0, st>>>(stats, TXS_STATS_LEN, 0);
+    if (num_unq > 0) {
+        if (!counts) return TXS_ERR_INVALID_ARG;
+        counts_from_presum_kernel<<<dim3(blocks_for(num_unq)), dim3(kThreads), 0, st>>>(
+            preSum, (int)num_unq, counts);
+    }
+    return status_of(hipGetLastError());
+}
+
+int txs_plan_seg_from_presum(const int32_t *preSum, int64_t num_total, int64_t num_unq,
+                             const int32_t *slot_of, int32_t *seg, void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_unq)) return TXS_ERR_INVALID_ARG;
+    if (num_total == 0) return TXS_OK;
+    if (!preSum || !slot_of || !seg || num_unq <= 0) return TXS_ERR_INVALID_ARG;
+    seg_from_presum_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+        preSum, num_total, (int)num_unq, slot_of, seg);
+    return status_of(hipGetLastError());
+}
+
+int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *perm,
+                        const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
+                        const int32_t *heavy_ids, int64_t num_special, void *scratch, void *out,
+                        int32_t *arg, int64_t num_total, int64_t channel, int64_t num_unq,
+                        void *stream) {
+    if (op != TXS_SUM && op != TXS_MEAN && op != TXS_MAX) return TXS_ERR_UNSUPPORTED;
+    if (dtype != TXS_F32 && dtype != TXS_F16 && dtype != TXS_BF16) return TXS_ERR_UNSUPPORTED;
+    if (!fits_i32(num_total) || !fits_i32(num_unq) || !fits_i32(channel) || num_special < 0 ||
+        num_special > num_unq)
+        return TXS_ERR_INVALID_ARG;
+    if (num_unq == 0 || channel == 0) return TXS_OK;
+    if (!out || !preSum || (op == TXS_MAX && !arg)) return TXS_ERR_INVALID_ARG;
+    if (num_total > 0 && (!feats || !seg || !slot_of)) return TXS_ERR_INVALID_ARG;
+    if (num_special > 0 && (!scratch || !heavy_ids)) return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const int N = (int)num_total, C = (int)channel, U = (int)num_unq;
+    const int elem = dtype == TXS_F32 ? 4 : 2;
+    hipError_t e = hipSuccess;
+    if (N > 0) {
+        Geometry geo = make_geometry(N, C, elem, feats, out, nullptr, op == TXS_MAX, arg);
+        if (dtype == TXS_F32)
+            e = launch_fwd<F32>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U);
+        else if (dtype == TXS_F16)
+            e = launch_fwd<F16>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U);
+        else
+            e = launch_fwd<BF16>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U);
+        if (e != hipSuccess) return TXS_ERR_LAUNCH;
+    }
+    if (num_special > 0) {
+        if (dtype == TXS_F32)
+            e = launch_finalize<F32>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U);
+        else if (dtype == TXS_F16)
+            e = launch_finalize<F16>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U);
+        else
+            e = launch_finalize<BF16>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U);
+    }
+    return status_of(e);
+}
+
+int txs_scatter_backward(int op, int dtype, const void *grad_out, const int32_t *arg,
+                         const int32_t *perm, const int32_t *seg, const int32_t *preSum,
+                         void *grad_in, int64_t num_total, int64_t channel, int64_t num_unq,
+                         void *stream) {
+    if (op != TXS_SUM && op != TXS_MEAN && op != TXS_MAX) return TXS_ERR_UNSUPPORTED;
+    if (dtype != TXS_F32 && dtype != TXS_F16 && dtype != TXS_BF16) return TXS_ERR_UNSUPPORTED;
+    if (!fits_i32(num_total) || !fits_i32(num_unq) || !fits_i32(channel)) return TXS_ERR_INVALID_ARG;
+    if (num_total == 0 || channel == 0) return TXS_OK;
+    if (!grad_out || !seg || !grad_in || num_unq <= 0) return TXS_ERR_INVALID_ARG;
+    if (op == TXS_MAX && !arg) return TXS_ERR_INVALID_ARG;
+    if (op == TXS_MEAN && !preSum) return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const int N = (int)num_total, C = (int)channel, U = (int)num_unq;
+    const int elem = dtype == TXS_F32 ? 4 : 2;
+    Geometry geo = make_geometry(N, C, elem, grad_out, grad_in, nullptr, op == TXS_MAX, arg);
+    hipError_t e;
+    if (dtype == TXS_F32)
+        e = launch_bwd<F32>(op, geo, st, grad_out, arg, perm, seg, preSum, grad_in, N, C, U);
+    else if (dtype == TXS_F16)
+        e = launch_bwd<F16>(op, geo, st, grad_out, arg, perm, seg, preSum, grad_in, N, C, U);
+    else
+        e = launch_bwd<BF16>(op, geo, st, grad_out, arg, perm, seg, preSum, grad_in, N, C, U);
+    return status_of(e);
+}
+
+}  // extern "C"
