@@ -1,0 +1,189 @@
+#!/usr/bin/env python3
+"""Benchmark of the voxel scatter path on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic points:
+``scatter_mean`` forward+backward and ``scatter_max`` (+argmax) forward+backward,
+through the public Python API (autograd included), with ``ScatterData`` built
+beforehand (the reference's own timing also keeps ``ScatterData`` construction
+outside the timed region, ``test/test_scatter.py:24,38-44``).  The workload is the
+LiDAR-like sweep: N = 1,000,000 points, C = 128 fp32 features, 0.2 m voxels.
+Inputs are resident in HBM before the timed region starts.
+
+``value`` is points per second per operator pass: ``2 * N / t_step`` (each step
+pushes the N points through two operators' forward+backward).  Per-operator
+times, GB/s and roofline fractions are in ``per_op``.
+
+Prints ONE JSON line on stdout.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=10)
+    p.add_argument("--kernel-iters", type=int, default=50, help="launches per per-kernel timing loop")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--points", type=int, default=1_000_000)
+    p.add_argument("--channels", type=int, default=128)
+    return p.parse_args()
+
+
+def event_ms(fn, iters, warm=5):
+    """Average duration of ``fn`` over ``iters`` back-to-back calls, measured with
+    HIP events recorded on the stream the kernels are launched on."""
+    for _ in range(warm):
+        fn()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def cpu_baseline(w, g_mean, g_max):
+    """The same step with stock torch CPU ops (scatter_reduce / index_add / gather) on
+    the host cores: a bounded sample of the same workload."""
+    from oracle import torch_oracle as tor
+    threads = os.cpu_count() or 1
+    threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
+    torch.set_num_threads(threads)
+    tor.step_mean_max(w.feats, w.unq_inv, w.unq_cnts, g_mean, g_max)   # warm-up
+    iters, t0 = 0, time.perf_counter()
+    while iters < 3 or (time.perf_counter() - t0 < 10.0 and iters < 10):
+        tor.step_mean_max(w.feats, w.unq_inv, w.unq_cnts, g_mean, g_max)
+        iters += 1
+    dt = (time.perf_counter() - t0) / iters
+    return {"value": 2 * w.N / dt, "unit": "points/s", "cores": torch.get_num_threads(),
+            "kind": "port", "ms_per_step": dt * 1e3,
+            "sample": f"{iters} full steps (N={w.N}, C={w.C}) of torch.scatter_reduce/index_add/gather on CPU"}
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    import torchex_amd as T
+    from torchex_amd import workloads
+    from torchex_amd._native import scatter_ext
+
+    dev = torch.device("cuda:0")
+    w = workloads.lidar_sweep(N=a.points, C=a.channels, seed=2)
+    N, C, U = w.N, w.C, w.U
+    g_mean_cpu = workloads.upstream_grad(U, C, 102)
+    g_max_cpu = workloads.upstream_grad(U, C, 103)
+
+    feats = w.feats.to(dev).requires_grad_(True)
+    inv, cnts = w.unq_inv.to(dev), w.unq_cnts.to(dev)
+    g_mean, g_max = g_mean_cpu.to(dev), g_max_cpu.to(dev)
+
+    # index preparation, timed separately
+    data = T.ScatterData(inv, cnts)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        data = T.ScatterData(inv, cnts)
+    torch.cuda.synchronize()
+    prep_ms = (time.perf_counter() - t0) / 5 * 1e3
+
+    def step():
+        feats.grad = None
+        T.scatter_mean(feats, data).backward(g_mean)
+        feats.grad = None
+        mx, _ = T.scatter_max(feats, data)
+        mx.backward(g_max)
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / a.steps * 1e3
+
+    # per-kernel durations: HIP events around back-to-back launches of one entry point
+    f = feats.detach()
+    sc = data.scratch(C)
+    plan = (data.perm, data.seg, data.preSum, data.slot_of, data.heavy_ids, sc)
+    _, arg = scatter_ext.forward(scatter_ext.MAX, f, *plan)
+    it = a.kernel_iters
+    kt = {
+        "mean_fwd": event_ms(lambda: scatter_ext.forward(scatter_ext.MEAN, f, *plan), it),
+        "mean_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MEAN, g_mean, None, data.perm, data.seg,
+                                                          data.preSum, N), it),
+        "max_fwd": event_ms(lambda: scatter_ext.forward(scatter_ext.MAX, f, *plan), it),
+        "max_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MAX, g_max, arg, data.perm, data.seg,
+                                                         data.preSum, N), it),
+        "sum_fwd": event_ms(lambda: scatter_ext.forward(scatter_ext.SUM, f, *plan), it),
+        "sum_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.SUM, g_mean, None, data.perm, data.seg,
+                                                         data.preSum, N), it),
+    }
+    ab = {k: workloads.algorithmic_bytes(k, N, C, U) for k in kt}
+    per_kernel = {k: {"ms": kt[k], "GBps": ab[k] / kt[k] / 1e6, "frac": ab[k] / kt[k] / 1e6 / HBM_PEAK_GBPS}
+                  for k in kt}
+    per_op = {}
+    for op in ("mean", "max", "sum"):
+        t = kt[op + "_fwd"] + kt[op + "_bwd"]
+        b = ab[op + "_fwd"] + ab[op + "_bwd"]
+        per_op[op] = {"ms_fwd": kt[op + "_fwd"], "ms_bwd": kt[op + "_bwd"], "points_per_s": N / t * 1e3,
+                      "GBps": b / t / 1e6, "frac_of_hbm_peak": b / t / 1e6 / HBM_PEAK_GBPS}
+
+    # a plain device copy of the feature matrix on the same box: the practical ceiling
+    dst = torch.empty_like(f)
+    copy_ms = event_ms(lambda: dst.copy_(f), 20)
+    copy_gbps = 2 * f.numel() * 4 / copy_ms / 1e6
+
+    dom = max(("max_fwd", "max_bwd", "mean_fwd", "mean_bwd"), key=lambda k: kt[k])
+    kname = {"max_fwd": "scatter_fwd_kernel<F32,4,MAX>", "mean_fwd": "scatter_fwd_kernel<F32,4,MEAN>",
+             "max_bwd": "scatter_bwd_kernel<F32,4,MAX>", "mean_bwd": "scatter_bwd_kernel<F32,4,MEAN>"}[dom]
+    roofline = {"bound": "hbm", "kernel": kname, "achieved": per_kernel[dom]["GBps"], "peak": HBM_PEAK_GBPS,
+                "unit": "GB/s", "frac": per_kernel[dom]["frac"], "traffic": None,
+                "algorithmic_bytes": ab[dom], "launch_ms": kt[dom]}
+
+    out = {
+        "metric": "scatter_mean+scatter_max(+argmax) fwd+bwd points/s (per operator pass), 1 GPU",
+        "value": 2 * N / ms_per_step * 1e3,
+        "unit": "points/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "lidar_sweep N=%d C=%d fp32, voxel 0.2m, U=%d, max_cnt=%d, unsorted unq_inv"
+                               % (N, C, U, data.max_cnt),
+                   "num_special_voxels": data.num_special, "heavy_threshold": data.heavy_threshold},
+        "roofline": roofline,
+        "per_op": per_op,
+        "per_kernel": per_kernel,
+        "device_copy_GBps": copy_gbps,
+        "index_prep_ms": prep_ms,
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w, g_mean_cpu, g_max_cpu)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

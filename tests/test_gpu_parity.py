@@ -1,0 +1,489 @@
+"""GPU parity: the HIP path (through scatter_ext -> C ABI) against the CPU oracle on
+identical seeded inputs.
+
+Bars: preSum / perm / counts / arg bit-exact; max values bit-exact; backward of sum,
+mean and max bit-exact (copies and one correctly rounded division); forward sum and
+mean within RTOL of the fp64 oracle, measured against the magnitude of the summands:
+``|got - want| <= RTOL * sum_i |x_i|`` (``/ cnt`` for mean), RTOL = 1e-5 for fp32 and
+2e-3 for fp16 / bf16 (fp32 accumulation).  A sum of zero-mean data has no meaningful
+relative error against its own (possibly tiny) value, hence the summand scale.
+For half-precision outputs the final rounding of the fp32 accumulator to the output
+dtype adds up to half a unit in the last place of that dtype (2^-11 relative for fp16,
+2^-8 for bf16 -- the latter alone is above 2e-3), so ``OUT_EPS * |want|`` is added.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as orc
+from torchex_amd import workloads
+
+pytestmark = pytest.mark.gpu
+
+RTOL = {torch.float32: 1e-5, torch.float16: 2e-3, torch.bfloat16: 2e-3}
+OUT_EPS = {torch.float32: 0.0, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}
+DEV = "cuda:0"
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def tx():
+    import torchex_amd
+    return torchex_amd
+
+
+def bits_equal(a, b):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    both_nan = np.isnan(a) & np.isnan(b)
+    return a.shape == b.shape and np.array_equal(a.view(np.uint32)[~both_nan], b.view(np.uint32)[~both_nan])
+
+
+def run_case(name, feats, unq_inv, unq_cnts, dtype=torch.float32, grad_seed=100, check_plan=True,
+             heavy_threshold=None):
+    """feats fp32 CPU [N, C]; unq_inv int64 CPU; unq_cnts int64 CPU.  Returns the
+    ScatterData for extra checks."""
+    T = tx()
+    N, C = feats.shape
+    U = unq_cnts.shape[0]
+    say(f"[case] {name} N={N} C={C} U={U} dtype={dtype}")
+    f_in = feats.to(dtype)                 # what both sides see
+    f32 = f_in.float().numpy()             # exact upcast for the oracle
+    inv32 = unq_inv.numpy().astype(np.int32)
+    cnt = unq_cnts.numpy()
+
+    fg = f_in.to(DEV).requires_grad_(True)
+    data = T.ScatterData(unq_inv.to(DEV), unq_cnts.to(DEV), heavy_threshold=heavy_threshold)
+
+    # ---- index preparation: integers, exact
+    want_pre = orc.presum(orc.counts(inv32, U))
+    assert np.array_equal(data.preSum.cpu().numpy(), want_pre), "preSum"
+    assert data.num_unq == U and data.max_cnt == (int(cnt.max()) if U else 0)
+    if check_plan and N:
+        want_perm = orc.stable_perm(inv32, want_pre)
+        got_perm = data.perm.cpu().numpy() if data.perm is not None else np.arange(N, dtype=np.int32)
+        assert np.array_equal(got_perm, want_perm), "perm"
+        seg = data.seg.cpu().numpy()
+        assert np.array_equal(seg & 0x7fffffff, inv32[want_perm]), "seg ids"
+        special = (cnt > data.heavy_threshold) | (cnt == 0)
+        assert np.array_equal(seg < 0, special[inv32[want_perm]]), "seg special bit"
+        assert data.num_special == int(special.sum())
+
+    # ---- forward
+    s = T.scatter_sum(fg, data)
+    mean = T.scatter_mean(fg, data)
+    mx, arg = T.scatter_max(fg, data)
+    assert s.dtype == dtype and mean.dtype == dtype and mx.dtype == dtype and arg.dtype == torch.int32
+    assert tuple(s.shape) == (U, C) and tuple(arg.shape) == (U, C)
+
+    s64 = orc.scatter_sum_f64(f32, inv32, U)
+    sabs = orc.scatter_sum_f64(np.abs(f32), inv32, U)
+    rt, oe = RTOL[dtype], OUT_EPS[dtype]
+    got = s.detach().float().cpu().numpy().astype(np.float64)
+    finite = np.isfinite(sabs)
+    assert np.all(np.abs(got - s64)[finite] <= (rt * sabs + oe * np.abs(s64))[finite] + 1e-30), \
+        f"sum: worst {np.max((np.abs(got - s64) / (sabs + 1e-30))[finite]):.3e}"
+    nz = cnt > 0
+    gotm = mean.detach().float().cpu().numpy().astype(np.float64)
+    wantm = s64[nz] / cnt[nz, None]
+    fm = finite[nz]
+    assert np.all(np.abs(gotm[nz] - wantm)[fm] <=
+                  (rt * sabs[nz] / cnt[nz, None] + oe * np.abs(wantm))[fm] + 1e-30), "mean"
+    assert np.all(np.isnan(gotm[~nz])), "mean of an empty voxel is 0/0 as in the reference"
+
+    want_max, want_arg = orc.scatter_max_first(f32, inv32, U)
+    got_arg = arg.cpu().numpy()
+    assert np.array_equal(got_arg, want_arg), \
+        f"arg: {int((got_arg != want_arg).sum())} of {want_arg.size} differ"
+    got_max = mx.detach().float().cpu().numpy()
+    if dtype == torch.float32:
+        assert bits_equal(got_max, want_max), "max"
+    else:  # lowest finite value of the dtype stands in for -FLT_MAX on winner-less cells
+        has = want_arg >= 0
+        assert bits_equal(got_max[has], want_max[has]), "max"
+        assert np.all(got_max[~has] == float(torch.finfo(dtype).min))
+
+    # ---- backward (upstream gradients N(0,1), rounded to the dtype)
+    g = workloads.upstream_grad(U, C, grad_seed).to(dtype)
+    g32 = g.float().numpy()
+    gd = g.to(DEV)
+
+    def grad_of(out):
+        fg.grad = None
+        out.backward(gd)
+        return fg.grad.detach().float().cpu().numpy()
+
+    assert bits_equal(grad_of(s), orc.sum_backward(g32, inv32)), "sum backward"
+    want_mb = orc.mean_backward(g32, np.maximum(cnt, 1), inv32)
+    if dtype != torch.float32:
+        want_mb = torch.from_numpy(want_mb).to(dtype).float().numpy()
+    assert bits_equal(grad_of(mean), want_mb), "mean backward"
+    assert bits_equal(grad_of(mx), orc.max_backward(g32, want_arg, N)), "max backward"
+    return data
+
+
+# ------------------------------------------------------------ tiny and edges --
+
+def test_hand_cases(hand_cases):
+    T = tx()
+    for c in hand_cases:
+        say("[case] hand", c["name"])
+        inv = torch.from_numpy(c["inv"]).long()
+        U = int(inv.max()) + 1
+        cnts = torch.bincount(inv, minlength=U)
+        f = torch.from_numpy(c["feats"]).to(DEV)
+        data = T.ScatterData(inv.to(DEV), cnts.to(DEV))
+        mx, arg = T.scatter_max(f, data)
+        assert bits_equal(mx.cpu().numpy(), c["max"]) and np.array_equal(arg.cpu().numpy(), c["arg"])
+        if "sum" in c:
+            np.testing.assert_allclose(T.scatter_sum(f, data).cpu().numpy(), c["sum"], rtol=1e-6)
+            np.testing.assert_allclose(T.scatter_mean(f, data).cpu().numpy(), c["mean"], rtol=1e-6)
+
+
+@pytest.mark.parametrize("C", [1, 3, 13, 16, 32, 64, 128, 129, 260])
+def test_channel_widths(C):
+    g = torch.Generator().manual_seed(C)
+    N, U = 3000, 97
+    inv = torch.randint(0, U, (N,), generator=g)
+    inv[:U] = torch.arange(U)
+    run_case(f"channels{C}", torch.randn((N, C), generator=g), inv, torch.bincount(inv, minlength=U))
+
+
+def test_single_voxel_single_point_and_singletons():
+    g = torch.Generator().manual_seed(1)
+    run_case("N1", torch.randn((1, 8), generator=g), torch.zeros(1, dtype=torch.long), torch.ones(1, dtype=torch.long))
+    run_case("U1", torch.randn((500, 8), generator=g), torch.zeros(500, dtype=torch.long),
+             torch.full((1,), 500, dtype=torch.long))
+    inv = torch.randperm(777, generator=g)
+    run_case("singletons", torch.randn((777, 12), generator=g), inv, torch.ones(777, dtype=torch.long))
+
+
+def test_heavy_ties_integers():
+    # small integer features: many equal maxima (first row must win), exact sums
+    g = torch.Generator().manual_seed(2)
+    N, U, C = 40000, 50, 20
+    inv = torch.randint(0, U, (N,), generator=g)
+    inv[:U] = torch.arange(U)
+    feats = torch.randint(-3, 4, (N, C), generator=g).float()
+    data = run_case("ties", feats, inv, torch.bincount(inv, minlength=U))
+    assert data.num_special == U  # ~800 rows per voxel: all go through the atomic table
+    T = tx()
+    s = T.scatter_sum(feats.to(DEV), data).cpu().numpy().astype(np.float64)
+    assert np.array_equal(s, orc.scatter_sum_f64(feats.numpy(), inv.numpy().astype(np.int32), U))
+
+
+def test_all_equal_features_pure_tie():
+    N, U, C = 5000, 9, 8
+    inv = torch.arange(N) % U
+    run_case("all_equal", torch.full((N, C), 2.5), inv, torch.bincount(inv, minlength=U))
+
+
+def test_special_values():
+    g = torch.Generator().manual_seed(3)
+    N, U, C = 6000, 40, 8
+    inv = torch.randint(0, U, (N,), generator=g)
+    inv[:U] = torch.arange(U)
+    f = torch.randn((N, C), generator=g)
+    f[torch.rand((N, C), generator=g) < 0.05] = float("nan")
+    f[torch.rand((N, C), generator=g) < 0.05] = float("-inf")
+    f[torch.rand((N, C), generator=g) < 0.02] = float("inf")
+    f[torch.rand((N, C), generator=g) < 0.05] = -0.0
+    f[torch.rand((N, C), generator=g) < 0.05] = 0.0
+    # voxels 0..2: only NaN / only -inf / NaN then -inf, light and heavy variants below
+    f[inv == 0] = float("nan")
+    f[inv == 1] = float("-inf")
+    f[inv == 2] = float("nan")
+    rows2 = torch.nonzero(inv == 2).flatten()
+    f[rows2[len(rows2) // 2:]] = float("-inf")
+    T = tx()
+    for thr in (None, 1 << 20):   # through the atomic table, and all in registers
+        say("[case] special values, heavy_threshold", thr)
+        data = T.ScatterData(inv.to(DEV), torch.bincount(inv, minlength=U).to(DEV), heavy_threshold=thr)
+        mx, arg = T.scatter_max(f.to(DEV), data)
+        wm, wa = orc.scatter_max_first(f.numpy(), inv.numpy().astype(np.int32), U)
+        assert np.array_equal(arg.cpu().numpy(), wa)
+        assert bits_equal(mx.cpu().numpy(), wm)
+        assert (wa[0] == -1).all() and (wa[1] == int(torch.nonzero(inv == 1)[0])).all()
+        # sums propagate NaN/inf like any fp32 sum
+        s = T.scatter_sum(f.to(DEV), data).cpu().numpy()
+        w = orc.scatter_sum_f64(f.numpy(), inv.numpy().astype(np.int32), U)
+        assert np.array_equal(np.isnan(s), np.isnan(w))
+        assert np.array_equal(np.isinf(s), np.isinf(w))
+
+
+def test_sorted_input_takes_identity_path_and_matches_unsorted():
+    T = tx()
+    g = torch.Generator().manual_seed(4)
+    N, U, C = 20000, 700, 32
+    inv = torch.randint(0, U, (N,), generator=g)
+    inv[:U] = torch.arange(U)
+    feats = torch.randn((N, C), generator=g)
+    order = torch.argsort(inv, stable=True)
+    d_sorted = run_case("sorted", feats[order], inv[order], torch.bincount(inv, minlength=U))
+    assert d_sorted.perm is None and d_sorted.is_sorted
+    d_uns = T.ScatterData(inv.to(DEV), torch.bincount(inv, minlength=U).to(DEV))
+    assert d_uns.perm is not None
+    a = T.scatter_max(feats[order].to(DEV), d_sorted)
+    b = T.scatter_max(feats.to(DEV), d_uns)
+    assert torch.equal(a[0], b[0])
+    assert torch.equal(order.to(DEV)[a[1].long()].int(), b[1])
+    # same accumulation order on both paths -> identical sums for the register path
+    sa = T.scatter_sum(feats[order].to(DEV), d_sorted)
+    sb = T.scatter_sum(feats.to(DEV), d_uns)
+    light = (torch.bincount(inv, minlength=U) <= d_uns.heavy_threshold).to(DEV)
+    assert torch.equal(sa[light], sb[light])
+    # mean is the sum divided once by the count (scatter_op.py:69)
+    m = T.scatter_mean(feats.to(DEV), d_uns)
+    assert torch.equal(m[light], (sb / d_uns.unq_cnts)[light])
+
+
+def test_empty_voxels_and_empty_input():
+    T = tx()
+    g = torch.Generator().manual_seed(5)
+    N, U, C = 1000, 30, 8
+    inv = torch.randint(0, U, (N,), generator=g)
+    inv[inv % 7 == 3] = 0   # leaves several ids unused
+    cnts = torch.bincount(inv, minlength=U)
+    assert (cnts == 0).any()
+    run_case("empty_voxels", torch.randn((N, C), generator=g), inv, cnts)
+    say("[case] N=0")
+    data = T.ScatterData(torch.zeros(0, dtype=torch.long, device=DEV), torch.zeros(4, dtype=torch.long, device=DEV))
+    f = torch.zeros((0, 8), device=DEV)
+    assert torch.equal(T.scatter_sum(f, data), torch.zeros((4, 8), device=DEV))
+    mx, arg = T.scatter_max(f, data)
+    assert (arg == -1).all() and (mx == torch.finfo(torch.float32).min).all()
+
+
+def test_heavy_threshold_boundary_runs():
+    # voxel sizes around the chunk length and the heavy threshold, in every phase
+    # relative to chunk boundaries
+    sizes = [1, 31, 32, 33, 63, 64, 65, 1, 2, 127, 128, 129, 64, 64, 1, 200, 32, 32, 32, 64, 1, 1, 65, 5]
+    sizes = sizes * 3 + [1] * 70 + [64] * 5 + [3] * 33
+    cnts = torch.tensor(sizes, dtype=torch.long)
+    U = len(sizes)
+    inv_sorted = torch.repeat_interleave(torch.arange(U), cnts)
+    g = torch.Generator().manual_seed(6)
+    N = int(cnts.sum())
+    feats = torch.randn((N, 16), generator=g)
+    run_case("boundaries_sorted", feats, inv_sorted, cnts)
+    p = torch.randperm(N, generator=g)
+    run_case("boundaries_shuffled", feats, inv_sorted[p], cnts)
+    run_case("boundaries_thr32", feats, inv_sorted[p], cnts, heavy_threshold=32)
+
+
+# ------------------------------------------------- the reference's own test --
+
+def test_reference_test_data_closed_forms(reference_counts):
+    """test/test_scatter.py: 500 sorted groups, each channel a permutation of 0..n-1:
+    sum = n(n-1)/2 exactly, mean = (n-1)/2 exactly, max = n-1, arg = its position."""
+    T = tx()
+    w = workloads.reference_test_groups(channel=128)
+    assert w.unq_cnts.tolist() == reference_counts["counts"] and w.N == 1229413
+    say("[case] reference test data", w.N, w.C)
+    n = w.unq_cnts.double()
+    col = w.feats[:, 0]
+    starts = torch.cumsum(w.unq_cnts, 0) - w.unq_cnts
+    argpos = torch.stack([s + torch.argmax(col[s:s + c]) for s, c in zip(starts.tolist(), w.unq_cnts.tolist())])
+    f = w.feats.to(DEV)
+    data = T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV))
+    assert data.max_cnt == 4996 and data.perm is None
+    assert data.preSum[-1].item() == w.N
+    for _ in range(2):
+        s = T.scatter_sum(f, data).cpu().double()
+        assert torch.equal(s, (n * (n - 1) / 2).unsqueeze(1).expand(-1, 128))
+        m = T.scatter_mean(f, data).cpu().double()
+        assert torch.equal(m, ((n - 1) / 2).unsqueeze(1).expand(-1, 128))
+        mx, arg = T.scatter_max(f, data)
+        assert torch.equal(mx.cpu().double(), (n - 1).unsqueeze(1).expand(-1, 128))
+        assert torch.equal(arg.cpu().long(), argpos.unsqueeze(1).expand(-1, 128))
+    # the reference module's own entry points on the same tensors (scatter.cpp:66-70)
+    import scatter_ext
+    pre = T.getPreSum(w.unq_inv.to(DEV))
+    assert torch.equal(pre, data.preSum)
+    out = f.new_zeros((w.U, 128))
+    scatter_ext.sum(f, pre, out, data.max_cnt)
+    assert torch.equal(out.cpu().double(), (n * (n - 1) / 2).unsqueeze(1).expand(-1, 128))
+    out = f.new_zeros((w.U, 128))
+    arg = pre.new_zeros((w.U, 128))
+    scatter_ext.max(f, pre, out, arg, data.max_cnt)
+    assert torch.equal(arg.cpu().long(), argpos.unsqueeze(1).expand(-1, 128))
+    assert torch.equal(out.cpu().double(), (n - 1).unsqueeze(1).expand(-1, 128))
+
+
+# ------------------------------------------------------- benchmark workloads --
+
+def test_uniform_box_and_reference_order_oracle():
+    w = workloads.uniform_box()
+    run_case("uniform_box", w.feats, w.unq_inv, w.unq_cnts)
+    # this workload also against the reference's own fp32 summation order
+    T = tx()
+    data = T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV))
+    s = T.scatter_sum(w.feats.to(DEV), data).cpu().numpy()
+    inv32 = w.unq_inv.numpy().astype(np.int32)
+    ref = orc.scatter_sum_reforder(w.feats.numpy(), inv32, w.U)
+    sabs = orc.scatter_sum_f64(np.abs(w.feats.numpy()), inv32, w.U)
+    assert np.all(np.abs(s.astype(np.float64) - ref) <= 1e-5 * sabs)
+    mr, ar = orc.scatter_max_reforder(w.feats.numpy(), inv32, w.U)
+    mx, arg = T.scatter_max(w.feats.to(DEV), data)
+    assert bits_equal(mx.cpu().numpy(), mr) and np.array_equal(arg.cpu().numpy(), ar)
+
+
+def test_lidar_sweep_fp32():
+    w = workloads.lidar_sweep()
+    run_case("lidar_sweep", w.feats, w.unq_inv, w.unq_cnts, grad_seed=102)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_lidar_sweep_half(dtype):
+    w = workloads.lidar_sweep(N=400_000, C=128, seed=2)
+    run_case("lidar_sweep_half", w.feats, w.unq_inv, w.unq_cnts, dtype=dtype, grad_seed=102)
+
+
+def test_zipf_contention():
+    w = workloads.zipf_contention()
+    assert int(w.unq_cnts.max()) > 100_000
+    run_case("zipf", w.feats, w.unq_inv, w.unq_cnts)
+
+
+def test_multi_sweep():
+    w = workloads.multi_sweep()
+    run_case("multi_sweep", w.feats, w.unq_inv, w.unq_cnts, check_plan=True)
+
+
+# ------------------------------------------------------ size-independent laws --
+
+def test_linearity_and_permutation_invariance_full_size():
+    T = tx()
+    w = workloads.lidar_sweep(N=1_000_000, C=32, seed=7)
+    say("[case] laws", w.N, w.C, w.U)
+    inv = w.unq_inv.to(DEV)
+    data = T.ScatterData(inv, w.unq_cnts.to(DEV))
+    f = w.feats.to(DEV)
+    mx, arg = T.scatter_max(f, data)
+    # arg points into the right voxel and at the winning value; no earlier row of the
+    # voxel attains it
+    assert torch.equal(inv[arg.long()], torch.arange(w.U, device=DEV).unsqueeze(1).expand(-1, w.C))
+    assert torch.equal(torch.gather(f, 0, arg.long()), mx)
+    assert (f <= mx[inv]).all()
+    rows = torch.arange(w.N, device=DEV).unsqueeze(1)
+    assert not ((f == mx[inv]) & (rows < arg[inv])).any()
+    # integer-valued features: sums are exact, so linearity and shuffling are bit-exact
+    fi = torch.randint(-8, 9, (w.N, w.C), generator=torch.Generator().manual_seed(1)).float().to(DEV)
+    fj = torch.randint(-8, 9, (w.N, w.C), generator=torch.Generator().manual_seed(2)).float().to(DEV)
+    assert torch.equal(T.scatter_sum(fi + fj, data), T.scatter_sum(fi, data) + T.scatter_sum(fj, data))
+    p = torch.randperm(w.N, generator=torch.Generator().manual_seed(3)).to(DEV)
+    data_p = T.ScatterData(inv[p], w.unq_cnts.to(DEV))
+    assert torch.equal(T.scatter_sum(fi[p], data_p), T.scatter_sum(fi, data))
+    mp, ap = T.scatter_max(f[p], data_p)
+    assert torch.equal(mp, mx)
+    ones = torch.ones((w.N, w.C), device=DEV)
+    assert torch.equal(T.scatter_sum(ones, data), w.unq_cnts.to(DEV).float().unsqueeze(1).expand(-1, w.C))
+    # backward of sum then forward again is multiplication by the counts
+    g = torch.randint(-8, 9, (w.U, w.C), generator=torch.Generator().manual_seed(4)).float().to(DEV)
+    x = torch.zeros((w.N, w.C), device=DEV, requires_grad=True)
+    T.scatter_sum(x, data).backward(g)
+    assert torch.equal(T.scatter_sum(x.grad, data), g * data.unq_cnts)
+
+
+def test_repeatability():
+    T = tx()
+    w = workloads.lidar_sweep(N=300_000, C=64, seed=9)
+    data = T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV))
+    f = w.feats.to(DEV)
+    m0, a0 = T.scatter_max(f, data)
+    mean0 = T.scatter_mean(f, data)
+    light = (w.unq_cnts <= data.heavy_threshold).to(DEV)
+    for _ in range(5):
+        m1, a1 = T.scatter_max(f, data)
+        assert torch.equal(m0, m1) and torch.equal(a0, a1)
+        assert torch.equal(T.scatter_mean(f, data)[light], mean0[light])
+
+
+# --------------------------------------------------------------- error paths --
+
+def test_error_paths():
+    T = tx()
+    import scatter_ext
+    g = torch.Generator().manual_seed(8)
+    N, U, C = 100, 5, 8
+    inv = torch.randint(0, U, (N,), generator=g)
+    inv[:U] = torch.arange(U)
+    cnts = torch.bincount(inv, minlength=U)
+    data = T.ScatterData(inv.to(DEV), cnts.to(DEV))
+    f = torch.randn((N, C), generator=g)
+    with pytest.raises(RuntimeError):
+        T.scatter_sum(f, data)                                # CPU tensor (scatter.cpp:4-5)
+    with pytest.raises(RuntimeError):
+        T.scatter_sum(f.to(DEV).t().contiguous().t(), data)   # non-contiguous (scatter.cpp:6-7)
+    with pytest.raises(RuntimeError):
+        T.scatter_sum(f.double().to(DEV), data)               # unsupported dtype
+    with pytest.raises(RuntimeError):
+        T.scatter_max(f[:50].to(DEV), data)                   # row count mismatch
+    with pytest.raises(RuntimeError):
+        T.ScatterData((inv + 1).to(DEV), cnts.to(DEV))        # id out of range
+    with pytest.raises(AssertionError):
+        T.ScatterData(inv.to(DEV), (cnts + 1).to(DEV))        # counts are not the histogram
+    with pytest.raises(AssertionError):
+        T.ScatterData(inv.to(DEV).reshape(N, 1, 1), cnts.to(DEV))
+    out = torch.zeros((U, C), device=DEV)
+    with pytest.raises(RuntimeError):
+        scatter_ext.sum(f.to(DEV), data.preSum.long(), out, data.max_cnt)  # preSum dtype
+    with pytest.raises(RuntimeError):
+        scatter_ext.sum(f.to(DEV), data.preSum[:-1].contiguous(), out, data.max_cnt)
+    # a failed call leaves the device usable
+    assert torch.isfinite(T.scatter_sum(f.to(DEV), data)).all()
+
+
+def test_c_abi_direct_call():
+    """Calls libtorchex_scatter.so through ctypes with raw device pointers, the way a
+    non-torch host would bind it."""
+    import ctypes
+    from torchex_amd import _native
+    lib = _native.cabi()
+    T = tx()
+    g = torch.Generator().manual_seed(10)
+    N, U, C = 5000, 300, 32
+    inv = torch.randint(0, U, (N,), generator=g)
+    inv[:U] = torch.arange(U)
+    feats = torch.randn((N, C), generator=g)
+    data = T.ScatterData(inv.to(DEV), torch.bincount(inv, minlength=U).to(DEV))
+    f = feats.to(DEV)
+    out = torch.empty((U, C), device=DEV)
+    arg = torch.empty((U, C), device=DEV, dtype=torch.int32)
+    scratch = torch.zeros((max(data.num_special, 1) * C,), device=DEV, dtype=torch.int64)
+    vp = ctypes.c_void_p
+    i64 = ctypes.c_int64
+    stream = vp(torch.cuda.current_stream().cuda_stream)
+    lib.txs_scatter_forward.restype = ctypes.c_int
+    rc = lib.txs_scatter_forward(
+        ctypes.c_int(2), ctypes.c_int(0), vp(f.data_ptr()), vp(data.perm.data_ptr()), vp(data.seg.data_ptr()),
+        vp(data.preSum.data_ptr()), vp(data.slot_of.data_ptr()),
+        vp(data.heavy_ids.data_ptr() if data.num_special else 0), i64(data.num_special), vp(scratch.data_ptr()),
+        vp(out.data_ptr()), vp(arg.data_ptr()), i64(N), i64(C), i64(U), stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    wm, wa = orc.scatter_max_first(feats.numpy(), inv.numpy().astype(np.int32), U)
+    assert bits_equal(out.cpu().numpy(), wm) and np.array_equal(arg.cpu().numpy(), wa)
+    assert (scratch == 0).all()
+    gin = torch.empty((N, C), device=DEV)
+    gup = torch.randn((U, C), generator=g).to(DEV)
+    lib.txs_scatter_backward.restype = ctypes.c_int
+    rc = lib.txs_scatter_backward(
+        ctypes.c_int(2), ctypes.c_int(0), vp(gup.data_ptr()), vp(arg.data_ptr()), vp(data.perm.data_ptr()),
+        vp(data.seg.data_ptr()), vp(data.preSum.data_ptr()), vp(gin.data_ptr()), i64(N), i64(C), i64(U), stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert bits_equal(gin.cpu().numpy(), orc.max_backward(gup.cpu().numpy(), wa, N))
+    # argument validation returns a status instead of launching
+    rc = lib.txs_scatter_forward(
+        ctypes.c_int(7), ctypes.c_int(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0), vp(0),
+        i64(N), i64(C), i64(U), stream)
+    assert rc == 3
+    rc = lib.txs_scatter_forward(
+        ctypes.c_int(0), ctypes.c_int(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0), vp(0),
+        i64(N), i64(C), i64(U), stream)
+    assert rc == 1

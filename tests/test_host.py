@@ -1,0 +1,126 @@
+"""CPU-side checks: the C ABI library loads and exports what the header declares,
+host-only entry points behave, the package imports, workloads are deterministic."""
+import ctypes
+import io
+import os
+import re
+from contextlib import redirect_stdout
+
+import numpy as np
+import torch
+
+from tests.conftest import ROOT
+from torchex_amd import workloads
+
+
+def _lib():
+    from torchex_amd import _native
+    return _native.cabi()
+
+
+def test_header_symbols_are_exported():
+    with open(os.path.join(ROOT, "include", "torchex_scatter.h")) as f:
+        text = f.read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(txs_[a-z_0-9]+)\s*\(", text)))
+    assert len(names) >= 15
+    lib = _lib()
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_host_only_entry_points():
+    lib = _lib()
+    assert lib.txs_abi_version() == 1
+    lib.txs_status_string.restype = ctypes.c_char_p
+    assert lib.txs_status_string(0) == b"ok"
+    assert b"invalid" in lib.txs_status_string(1)
+    assert b"unknown" in lib.txs_status_string(99)
+    assert lib.txs_default_heavy_threshold() >= lib.txs_chunk_rows() > 0
+    lib.txs_scan_workspace_len.restype = ctypes.c_int64
+    lib.txs_sort_workspace_len.restype = ctypes.c_int64
+    assert lib.txs_scan_workspace_len(ctypes.c_int64(0)) >= 1
+    n = 1_000_000
+    assert lib.txs_sort_workspace_len(ctypes.c_int64(n), ctypes.c_int64(120000)) >= 2 * n
+
+
+def test_argument_validation_needs_no_gpu():
+    # these return before any launch
+    lib = _lib()
+    vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    rc = lib.txs_scatter_forward(ci(9), ci(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0),
+                                 vp(0), i64(1), i64(1), i64(1), vp(0))
+    assert rc == 3
+    rc = lib.txs_scatter_forward(ci(0), ci(5), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0),
+                                 vp(0), i64(1), i64(1), i64(1), vp(0))
+    assert rc == 3
+    rc = lib.txs_scatter_forward(ci(0), ci(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0),
+                                 vp(0), i64(1 << 40), i64(1), i64(1), vp(0))
+    assert rc == 1
+    rc = lib.txs_scatter_backward(ci(2), ci(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(5), i64(4), i64(2),
+                                  vp(0))
+    assert rc == 1
+    rc = lib.txs_get_presum(vp(0), vp(0), i64(-1), i64(0), vp(0))
+    assert rc == 1
+
+
+def test_package_surface_matches_reference_exports():
+    import torchex
+    import torchex_amd
+    for name in ["scatter_sum", "scatter_mean", "scatter_max", "ScatterData", "TorchTimer"]:
+        assert hasattr(torchex, name) and getattr(torchex, name) is getattr(torchex_amd, name)
+    import scatter_ext
+    for name in ["sum", "max", "getPreSum"]:   # torchex/src/scatter/scatter.cpp:66-70
+        assert callable(getattr(scatter_ext, name))
+
+
+def test_cpu_tensors_are_rejected_not_silently_computed():
+    import pytest
+    import scatter_ext
+    f = torch.zeros((4, 4))
+    pre = torch.tensor([0, 4], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        scatter_ext.sum(f, pre, torch.zeros((1, 4)), 4)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        scatter_ext.getPreSum(torch.zeros(4, dtype=torch.int32), pre)
+
+
+def test_torch_timer_prints_running_mean():
+    from torchex_amd import TorchTimer
+    t = TorchTimer(2)
+    buf = io.StringIO()
+    with redirect_stdout(buf):
+        for _ in range(4):
+            with t.timing("x"):
+                pass
+        with t.timing("off", freq=-1):
+            pass
+    lines = buf.getvalue().strip().splitlines()
+    assert len(lines) == 2 and all(l.startswith("Average time cost of x:") and l.endswith("ms") for l in lines)
+
+
+def test_workloads_are_seeded_and_shaped():
+    a = workloads.uniform_box(N=5000, C=4)
+    b = workloads.uniform_box(N=5000, C=4)
+    assert torch.equal(a.feats, b.feats) and torch.equal(a.unq_inv, b.unq_inv)
+    assert a.unq_cnts.sum().item() == 5000 and a.unq_inv.max().item() == a.U - 1
+    w = workloads.lidar_sweep(N=20000, C=4)
+    assert w.unq_cnts.sum().item() == 20000
+    z = workloads.zipf_contention(N=20000, C=2, num_ids=64)
+    assert z.U <= 64 and z.unq_cnts.max().item() > 20000 / 64
+    m = workloads.multi_sweep(N_per=2000, sweeps=3, C=2)
+    assert m.N == 6000
+    # keys of different sweeps never collide: every voxel's rows come from one sweep
+    sweep = torch.arange(6000) // 2000
+    lo = torch.full((m.U,), 99).scatter_reduce(0, m.unq_inv, sweep, "amin")
+    hi = torch.full((m.U,), -1).scatter_reduce(0, m.unq_inv, sweep, "amax")
+    assert torch.equal(lo, hi)
+
+
+def test_algorithmic_bytes_formulae():
+    N, C, U = 1_000_000, 128, 120_000
+    assert workloads.algorithmic_bytes("max_fwd", N, C, U) == N * C * 4 + 4 * N + U * C * 4 + 4 * U * C
+    fb = workloads.algorithmic_bytes("max_fwd", N, C, U) + workloads.algorithmic_bytes("max_bwd", N, C, U)
+    assert abs(fb - 1.278e9) / 1.278e9 < 0.01
+    fb = workloads.algorithmic_bytes("mean_fwd", N, C, U) + workloads.algorithmic_bytes("mean_bwd", N, C, U)
+    assert abs(fb - 1.157e9) / 1.157e9 < 0.01

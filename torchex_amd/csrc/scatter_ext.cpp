@@ -11,8 +11,10 @@
 
 #include <torch/extension.h>
 
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+// PyTorch-ROCm keeps the device type spelled "cuda"; these are its HIP guard
+// and stream accessors for that spelling.
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <optional>
 #include <tuple>
@@ -51,7 +53,7 @@ void check_status(int st, const char *what) {
 }
 
 void *cur_stream(const Tensor &x) {
-    return (void *)c10::hip::getCurrentHIPStream(x.device().index()).stream();
+    return (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(x.device().index()).stream();
 }
 
 const int32_t *i32p(const Tensor &x) { return x.numel() ? x.data_ptr<int32_t>() : nullptr; }
@@ -95,7 +97,7 @@ std::tuple<Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>> buil
     check_i32(unq_inv, "unq_inv");
     TORCH_CHECK(unq_inv.dim() == 1, "unq_inv must be 1-D");
     TORCH_CHECK(num_unq >= 0, "num_unq must be non-negative");
-    c10::hip::HIPGuard guard(unq_inv.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(unq_inv.device());
     const int64_t N = unq_inv.numel(), U = num_unq;
     Tensor counts = empty_i32(U, unq_inv);
     Tensor stats = empty_i32(TXS_STATS_LEN, unq_inv);
@@ -127,7 +129,7 @@ std::tuple<Tensor, Tensor, Tensor, std::vector<int64_t>> plan_from_presum(
     const Tensor &preSum, int64_t num_total, int64_t heavy_threshold) {
     check_i32(preSum, "preSum");
     TORCH_CHECK(preSum.dim() == 1 && preSum.numel() >= 1, "preSum must be 1-D with num_unq+1 entries");
-    c10::hip::HIPGuard guard(preSum.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(preSum.device());
     const int64_t U = preSum.numel() - 1, N = num_total;
     void *st = cur_stream(preSum);
     Tensor counts = empty_i32(U, preSum);
@@ -185,7 +187,7 @@ std::tuple<Tensor, OptTensor> forward(int64_t op, const Tensor &feats, const Opt
     check_dev(scratch, "scratch");
     TORCH_CHECK(scratch.scalar_type() == at::kLong, "scratch must be int64");
     TORCH_CHECK(seg.device() == feats.device(), "plan and feats live on different devices");
-    c10::hip::HIPGuard guard(feats.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(feats.device());
     const int64_t C = feats.size(1), U = preSum.numel() - 1;
     Tensor out = at::empty({U, C}, feats.options());
     OptTensor arg;
@@ -211,7 +213,7 @@ Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const 
         check_i32(*arg, "arg");
         TORCH_CHECK(arg->dim() == 2 && arg->size(0) == U && arg->size(1) == C, "arg must be [num_unq, channel]");
     }
-    c10::hip::HIPGuard guard(grad_out.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(grad_out.device());
     const int dt = dtype_code(grad_out, "grad_out");
     Tensor gin = at::empty({N, C}, grad_out.options());
     void *st = cur_stream(grad_out);
@@ -234,7 +236,7 @@ void csr_reduce(int op, Tensor feats, Tensor preSum, Tensor out, OptTensor arg) 
     TORCH_CHECK(feats.dim() == 2 && out.dim() == 2, "feats and out must be 2-D");
     TORCH_CHECK(out.scalar_type() == feats.scalar_type(), "out dtype must match feats");
     TORCH_CHECK(preSum.numel() == out.size(0) + 1, "preSum must have out.size(0)+1 entries");
-    c10::hip::HIPGuard guard(feats.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(feats.device());
     auto [seg, slot_of, heavy_ids, hs] =
         plan_from_presum(preSum, feats.size(0), txs_default_heavy_threshold());
     Tensor scratch = make_scratch(heavy_ids.numel(), feats.size(1), feats);
@@ -257,7 +259,7 @@ void max_ref(Tensor feats, Tensor preSum, Tensor out, Tensor arg, int64_t /*max_
 void get_presum_ref(Tensor unq_inv, Tensor preSum) {
     check_i32(unq_inv, "unq_inv");
     check_i32(preSum, "preSum");
-    c10::hip::HIPGuard guard(unq_inv.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(unq_inv.device());
     check_status(txs_get_presum(i32p(unq_inv), i32w(preSum), unq_inv.numel(), preSum.numel(),
                                 cur_stream(unq_inv)),
                  "getPreSum");
