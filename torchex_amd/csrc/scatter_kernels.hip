@@ -29,9 +29,28 @@
 
 namespace {
 
+#ifndef TXS_CHUNK
+#define TXS_CHUNK 16
+#endif
+#ifndef TXS_BATCH
+#define TXS_BATCH 4
+#endif
+#ifndef TXS_NT_LOADS
+#define TXS_NT_LOADS 1
+#endif
+#ifndef TXS_NT_STORES
+#define TXS_NT_STORES 1
+#endif
+#ifndef TXS_DIAG
+#define TXS_DIAG 0
+#endif
+#ifndef TXS_NT_OUT
+#define TXS_NT_OUT 1
+#endif
+
 constexpr int kThreads = 256;        // 4 wavefronts per workgroup
-constexpr int kChunk = 32;           // sorted positions per lane group
-constexpr int kBatch = 8;            // rows in flight per lane group
+constexpr int kChunk = TXS_CHUNK;    // sorted positions per lane group
+constexpr int kBatch = TXS_BATCH;    // rows in flight per lane group
 constexpr int kHeavyDefault = 64;    // voxels above this many rows use the atomic path
 constexpr int kSpecialBit = (int)0x80000000;
 constexpr int kIdMask = 0x7fffffff;
@@ -82,11 +101,56 @@ __device__ __forceinline__ void st(T *p, const Pack<T, VEC> &x) {
     *reinterpret_cast<Pack<T, VEC> *>(p) = x;
 }
 
-// Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous
-// range of chunks so neighbouring chunks (which share voxels, seg/perm cache
-// lines and upstream-gradient rows) meet in the same L2.  gridDim.x is a
-// multiple of 8.
-__device__ __forceinline__ int xcd_block(int b, int nb) { return (b & 7) * (nb >> 3) + (b >> 3); }
+// Streaming variants: data touched exactly once (feature rows on the way in,
+// input-gradient rows on the way out) is moved with the non-temporal hint so it
+// does not evict the index arrays and upstream-gradient rows that are re-read.
+template <typename T, int VEC>
+struct VecOf {
+    typedef T type __attribute__((ext_vector_type(VEC)));
+};
+template <typename T>
+struct VecOf<T, 1> {
+    typedef T type;
+};
+template <typename T, int VEC>
+__device__ __forceinline__ Pack<T, VEC> ld_stream(const T *p) {
+#if TXS_NT_LOADS
+    using V = typename VecOf<T, VEC>::type;
+    V v = __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
+    Pack<T, VEC> r;
+    __builtin_memcpy(&r, &v, sizeof(r));
+    return r;
+#else
+    return ld<T, VEC>(p);
+#endif
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void st_stream(T *p, const Pack<T, VEC> &x) {
+#if TXS_NT_STORES
+    using V = typename VecOf<T, VEC>::type;
+    V v;
+    __builtin_memcpy(&v, &x, sizeof(v));
+    __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
+#else
+    st<T, VEC>(p, x);
+#endif
+}
+
+// Workgroups are handed to the 8 XCDs round-robin.  Tiles are dealt to the XCDs
+// in spans of kXcdSpan consecutive tiles so that neighbours (which share voxels
+// and upstream-gradient rows) can meet in one L2.  Handing each XCD one long
+// contiguous range instead was measured to be much slower on skewed data: bytes
+// per position vary along the sorted order, so the XCDs finish at different times.
+#ifndef TXS_XCD_SPAN
+#define TXS_XCD_SPAN 1
+#endif
+constexpr int kXcdSpan = TXS_XCD_SPAN;  // gridDim.x is a multiple of 8 * kXcdSpan
+__device__ __forceinline__ int xcd_block(int b, int nb) {
+    (void)nb;
+    if (kXcdSpan == 1) return b;
+    const int xcd = b & 7, q = b >> 3;
+    return (q / kXcdSpan) * (8 * kXcdSpan) + xcd * kXcdSpan + (q % kXcdSpan);
+}
 
 // Monotonic map from non-NaN floats to unsigned ints; -0.0 is folded into +0.0
 // first so the two zeros tie, as they do under the reference's float compare.
@@ -359,46 +423,89 @@ __global__ void seg_from_presum_kernel(const int *__restrict__ preSum, long n, i
 }
 
 // ----------------------------------------------------------------- forward --
+//
+// One workgroup owns a tile of G * kChunk consecutive sorted positions, where
+// G = 256 / (lanes per row) lane groups each own kChunk of them.  The tile's seg
+// and perm entries (plus one entry before and kMargin after) are staged in LDS
+// by one coalesced load, so the row loads that follow never wait on an index
+// load, and a lane group can look across its chunk borders for free.  Row loads
+// are double-buffered: the next batch is in flight while the current one is
+// reduced.
+
+constexpr int kMargin = 64;           // staged entries past the tile's end
+constexpr int kNoSeg = 0x7fffffff;    // never a valid seg value
 
 template <class TR, int VEC, int OP>
 __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     const typename TR::raw *__restrict__ feats, const int *__restrict__ perm,
-    const int *__restrict__ seg, const int *__restrict__ preSum, const int *__restrict__ slot_of,
+    const int *__restrict__ seg, const int *__restrict__ slot_of,
     typename TR::raw *__restrict__ out, int *__restrict__ arg,
-    unsigned long long *__restrict__ scratch, int N, int C, int U, int lpr_log2, int n_groups) {
+    unsigned long long *__restrict__ scratch, int N, int C, int U, int lpr_log2) {
     using raw = typename TR::raw;
-    const int group = xcd_block(blockIdx.x, gridDim.x) * (kThreads >> lpr_log2) +
-                      ((int)threadIdx.x >> lpr_log2);
-    const int col = ((int)blockIdx.y << lpr_log2 | ((int)threadIdx.x & ((1 << lpr_log2) - 1))) * VEC;
-    if (group >= n_groups || col >= C) return;
-
-    // Range of sorted positions [a, b) this lane group reduces: its chunk,
-    // minus the tail of an ordinary run that began in an earlier chunk, plus
-    // the tail of an ordinary run that begins here and ends later.
-    int a = group * kChunk;
-    const int chunk_end = min(N, a + kChunk);
-    {
-        int s0 = seg[a];
-        if (a > 0 && s0 >= 0 && seg[a - 1] == s0) a = preSum[s0 + 1];
+    extern __shared__ int lds[];
+    const int G = kThreads >> lpr_log2;
+    const int T = G * kChunk;
+    const int n_seg_s = T + kMargin + 1;  // positions t0-1 .. t0+T+kMargin-1
+    int *seg_s = lds;
+    int *perm_s = lds + n_seg_s;          // positions t0 .. t0+T+kMargin-1
+    const long t0l = (long)xcd_block(blockIdx.x, gridDim.x) * T;
+    if (t0l >= N) return;  // uniform for the workgroup
+    const int t0 = (int)t0l;
+    for (int e = threadIdx.x; e < n_seg_s; e += kThreads) {
+        const long p = (long)t0 - 1 + e;
+        const bool in = p >= 0 && p < N;
+        seg_s[e] = in ? seg[p] : kNoSeg;
+        if (e >= 1) perm_s[e - 1] = in ? (perm ? perm[p] : (int)p) : -1;
     }
-    if (a >= chunk_end) return;
-    int b = chunk_end;
-    if (chunk_end < N) {
-        int sl = seg[chunk_end - 1];
-        if (sl >= 0 && seg[chunk_end] == sl) b = min(N, preSum[sl + 1]);
+    __syncthreads();
+
+    const int col = ((int)blockIdx.y << lpr_log2 | ((int)threadIdx.x & ((1 << lpr_log2) - 1))) * VEC;
+    if (col >= C) return;
+    // l indexes seg_s (position t0 - 1 + l); entries past the staged range are
+    // fetched from global memory (only an ordinary run longer than kMargin that
+    // crosses the tile's end gets there)
+    auto seg_at = [&](int l) -> int {
+        if (l < n_seg_s) return seg_s[l];
+        const long p = (long)t0 - 1 + l;
+        return p < N ? seg[p] : kNoSeg;
+    };
+    auto row_at = [&](int l) -> int {
+        if (l < n_seg_s) return perm_s[l - 1];
+        const long p = (long)t0 - 1 + l;
+        return p < N ? (perm ? perm[p] : (int)p) : -1;
+    };
+
+    // Range [la, lb) this lane group reduces: its chunk, minus the tail of an
+    // ordinary run that began in an earlier chunk, plus the tail of an ordinary
+    // run that begins here and ends later.
+    int la = ((int)threadIdx.x >> lpr_log2) * kChunk + 1;
+    const int lend = min(la + kChunk, N - t0 + 1);
+    if (la >= lend) return;
+    {
+        const int s0 = seg_s[la];
+        if (s0 >= 0 && seg_s[la - 1] == s0) {
+            do ++la; while (la < lend && seg_s[la] == s0);
+            if (la >= lend) return;
+        }
+    }
+    int lb = lend;
+    {
+        const int sl = seg_s[lend - 1];
+        if (sl >= 0)
+            while (seg_at(lb) == sl) ++lb;  // ends at the latest at N (kNoSeg)
     }
 
     float acc[VEC];
     int idx[VEC];
-    int cur = seg[a];
-    int run_j0 = a;
+    int cur = seg_s[la];
+    int run_l0 = la;
 #pragma unroll
     for (int k = 0; k < VEC; ++k) {
         acc[k] = (OP == TXS_MAX) ? -__builtin_inff() : 0.0f;
         idx[k] = -1;
     }
 
-    // Emit the finished run [run_j0, run_end) of voxel `cur`.
+    // Emit the finished run [run_l0, run_end) of voxel `cur`.
     auto flush = [&](int run_end) {
         const int u = cur & kIdMask;
         if ((unsigned)u >= (unsigned)U) return;
@@ -409,8 +516,8 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
             if (__builtin_expect(missing, 0)) {
                 // No value above -inf was seen in some channel: the run holds
                 // only -inf and NaN there.  The first -inf row wins.
-                for (int p = run_j0; p < run_end; ++p) {
-                    int row = perm ? perm[p] : p;
+                for (int p = run_l0; p < run_end; ++p) {
+                    const int row = row_at(p);
                     if ((unsigned)row >= (unsigned)N) continue;
                     Pack<raw, VEC> x = ld<raw, VEC>(feats + (size_t)row * C + col);
 #pragma unroll
@@ -426,7 +533,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) r.v[k] = TR::from_f(acc[k]);
             } else if (OP == TXS_MEAN) {
-                const float d = (float)(run_end - run_j0);
+                const float d = (float)(run_end - run_l0);
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) r.v[k] = TR::from_f(acc[k] / d);
             } else {
@@ -436,9 +543,9 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                     r.v[k] = idx[k] >= 0 ? TR::from_f(acc[k]) : TR::lowest();
                     ai.v[k] = idx[k];
                 }
-                st<int, VEC>(arg + o, ai);
+                st_stream<int, VEC>(arg + o, ai);
             }
-            st<raw, VEC>(out + o, r);
+            st_stream<raw, VEC>(out + o, r);
         } else {  // heavy voxel: merge this chunk's partial into the scratch table
             const int slot = slot_of[u];
             if (slot < 0) return;
@@ -460,28 +567,31 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
         }
     };
 
-    for (int j = a; j < b; j += kBatch) {
+    struct Batch {
         int segs[kBatch], rows[kBatch];
         Pack<raw, VEC> v[kBatch];
+    };
+    auto issue = [&](Batch &bt, int l) {
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
-            const int jj = j + i;
-            const bool ok = jj < b;
-            const int js = ok ? jj : a;
-            segs[i] = seg[js];
-            int r = perm ? perm[js] : js;
-            rows[i] = (ok && (unsigned)r < (unsigned)N) ? r : -1;
+            const int ll = l + i;
+            const bool ok = ll < lb;
+            bt.segs[i] = ok ? seg_at(ll) : kNoSeg;
+            const int r = ok ? row_at(ll) : -1;
+            bt.rows[i] = ((unsigned)r < (unsigned)N) ? r : -1;
         }
 #pragma unroll
         for (int i = 0; i < kBatch; ++i)
-            if (rows[i] >= 0) v[i] = ld<raw, VEC>(feats + (size_t)rows[i] * C + col);
+            if (bt.rows[i] >= 0) bt.v[i] = ld_stream<raw, VEC>(feats + (size_t)bt.rows[i] * C + col);
+    };
+    auto consume = [&](const Batch &bt, int l) {
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
-            if (rows[i] < 0) continue;
-            if (segs[i] != cur) {
-                flush(j + i);
-                cur = segs[i];
-                run_j0 = j + i;
+            if (bt.rows[i] < 0) continue;
+            if (bt.segs[i] != cur) {
+                flush(l + i);
+                cur = bt.segs[i];
+                run_l0 = l + i;
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) {
                     acc[k] = (OP == TXS_MAX) ? -__builtin_inff() : 0.0f;
@@ -490,18 +600,33 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
             }
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
-                const float x = TR::to_f(v[i].v[k]);
+                const float x = TR::to_f(bt.v[i].v[k]);
                 if (OP == TXS_MAX) {
                     const bool take = x > acc[k];  // strict: first row wins ties, NaN never wins
                     acc[k] = take ? x : acc[k];
-                    idx[k] = take ? rows[i] : idx[k];
+                    idx[k] = take ? bt.rows[i] : idx[k];
                 } else {
                     acc[k] += x;
                 }
             }
         }
+    };
+
+    Batch b0, b1;
+    issue(b0, la);
+    for (int l = la;;) {
+        int ln = l + kBatch;
+        if (ln < lb) issue(b1, ln);
+        consume(b0, l);
+        if (ln >= lb) break;
+        l = ln;
+        ln = l + kBatch;
+        if (ln < lb) issue(b0, ln);
+        consume(b1, l);
+        if (ln >= lb) break;
+        l = ln;
     }
-    flush(b);
+    flush(lb);
 }
 
 // Turn the scratch table of the special voxels into output rows and clear it.
@@ -539,69 +664,116 @@ __global__ void scatter_finalize_kernel(const typename TR::raw *__restrict__ fea
 }
 
 // ---------------------------------------------------------------- backward --
+//
+// Same tiling and LDS staging as the forward pass, no border logic: position j
+// writes row perm[j] of the input gradient from the upstream row of voxel
+// seg[j].  The upstream row (and arg row) is fetched once per run of equal ids
+// inside a chunk, and the fetches of the next batch are in flight while the
+// current batch is stored.
 
 template <class TR, int VEC, int OP>
 __global__ __launch_bounds__(kThreads) void scatter_bwd_kernel(
     const typename TR::raw *__restrict__ g, const int *__restrict__ arg,
     const int *__restrict__ perm, const int *__restrict__ seg, const int *__restrict__ preSum,
-    typename TR::raw *__restrict__ gin, int N, int C, int U, int lpr_log2, int n_groups) {
+    typename TR::raw *__restrict__ gin, int N, int C, int U, int lpr_log2) {
     using raw = typename TR::raw;
-    const int group = xcd_block(blockIdx.x, gridDim.x) * (kThreads >> lpr_log2) +
-                      ((int)threadIdx.x >> lpr_log2);
-    const int col = ((int)blockIdx.y << lpr_log2 | ((int)threadIdx.x & ((1 << lpr_log2) - 1))) * VEC;
-    if (group >= n_groups || col >= C) return;
-    const int a = group * kChunk;
-    const int b = min(N, a + kChunk);
+    extern __shared__ int lds[];
+    const int G = kThreads >> lpr_log2;
+    const int T = G * kChunk;
+    int *seg_s = lds;
+    int *perm_s = lds + T;
+    const long t0l = (long)xcd_block(blockIdx.x, gridDim.x) * T;
+    if (t0l >= N) return;  // uniform for the workgroup
+    const int t0 = (int)t0l;
+    for (int e = threadIdx.x; e < T; e += kThreads) {
+        const long p = (long)t0 + e;
+        const bool in = p < N;
+        const int u = in ? (seg[p] & kIdMask) : -1;
+        const int r = in ? (perm ? perm[p] : (int)p) : -1;
+        const bool good = (unsigned)u < (unsigned)U && (unsigned)r < (unsigned)N;
+        seg_s[e] = good ? u : -1;
+        perm_s[e] = good ? r : -1;
+    }
+    __syncthreads();
 
-    int cur = -1;  // voxel whose scaled gradient row is held in q (mean only)
-    Pack<raw, VEC> q;
-    for (int j = a; j < b; j += kBatch) {
+    const int col = ((int)blockIdx.y << lpr_log2 | ((int)threadIdx.x & ((1 << lpr_log2) - 1))) * VEC;
+    if (col >= C) return;
+    const int la = ((int)threadIdx.x >> lpr_log2) * kChunk;
+    const int lb = min(la + kChunk, N - t0);
+    if (la >= lb) return;
+
+    struct Batch {
         int us[kBatch], rows[kBatch];
+        bool need[kBatch];
         Pack<raw, VEC> gv[kBatch];
         Pack<int, VEC> av[kBatch];
         int c0[kBatch], c1[kBatch];
+    };
+    auto issue = [&](Batch &bt, int l) {
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
-            const int jj = j + i;
-            const bool ok = jj < b;
-            const int js = ok ? jj : a;
-            const int u = seg[js] & kIdMask;
-            const int r = perm ? perm[js] : js;
-            us[i] = u;
-            rows[i] = (ok && (unsigned)r < (unsigned)N && (unsigned)u < (unsigned)U) ? r : -1;
+            const int ll = l + i;
+            const bool ok = ll < lb;
+            bt.us[i] = ok ? seg_s[ll] : -1;
+            bt.rows[i] = ok ? perm_s[ll] : -1;
+            // first position of the chunk, or the voxel changes here
+            bt.need[i] = bt.rows[i] >= 0 && (ll == la || seg_s[ll - 1] != bt.us[i]);
         }
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
-            if (rows[i] < 0) continue;
-            const size_t o = (size_t)us[i] * C + col;
-            gv[i] = ld<raw, VEC>(g + o);
-            if (OP == TXS_MAX) av[i] = ld<int, VEC>(arg + o);
+            if (!bt.need[i]) continue;
+            const size_t o = (size_t)bt.us[i] * C + col;
+            bt.gv[i] = ld<raw, VEC>(g + o);
+            if (OP == TXS_MAX) bt.av[i] = ld<int, VEC>(arg + o);
             if (OP == TXS_MEAN) {
-                c0[i] = preSum[us[i]];
-                c1[i] = preSum[us[i] + 1];
+                bt.c0[i] = preSum[bt.us[i]];
+                bt.c1[i] = preSum[bt.us[i] + 1];
             }
         }
+    };
+    Pack<raw, VEC> q;   // (scaled) upstream row of the current voxel
+    Pack<int, VEC> aq;  // its arg row
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        q.v[k] = TR::zero();
+        aq.v[k] = -1;
+    }
+    auto consume = [&](const Batch &bt) {
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
-            if (rows[i] < 0) continue;
-            Pack<raw, VEC> r;
-            if (OP == TXS_SUM) {
-                r = gv[i];
-            } else if (OP == TXS_MEAN) {
-                if (us[i] != cur) {  // one division per run, not per row
-                    cur = us[i];
-                    const float d = (float)(c1[i] - c0[i]);
+            if (bt.rows[i] < 0) continue;
+            if (bt.need[i]) {
+                if (OP == TXS_MEAN) {  // one division per run, not per row
+                    const float d = (float)(bt.c1[i] - bt.c0[i]);
 #pragma unroll
-                    for (int k = 0; k < VEC; ++k) q.v[k] = TR::from_f(TR::to_f(gv[i].v[k]) / d);
+                    for (int k = 0; k < VEC; ++k) q.v[k] = TR::from_f(TR::to_f(bt.gv[i].v[k]) / d);
+                } else {
+                    q = bt.gv[i];
                 }
-                r = q;
-            } else {
-#pragma unroll
-                for (int k = 0; k < VEC; ++k)
-                    r.v[k] = (av[i].v[k] == rows[i]) ? gv[i].v[k] : TR::zero();
+                if (OP == TXS_MAX) aq = bt.av[i];
             }
-            st<raw, VEC>(gin + (size_t)rows[i] * C + col, r);
+            Pack<raw, VEC> r = q;
+            if (OP == TXS_MAX) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) r.v[k] = (aq.v[k] == bt.rows[i]) ? q.v[k] : TR::zero();
+            }
+            st_stream<raw, VEC>(gin + (size_t)bt.rows[i] * C + col, r);
         }
+    };
+
+    Batch b0, b1;
+    issue(b0, la);
+    for (int l = la;;) {
+        int ln = l + kBatch;
+        if (ln < lb) issue(b1, ln);
+        consume(b0);
+        if (ln >= lb) break;
+        l = ln;
+        ln = l + kBatch;
+        if (ln < lb) issue(b0, ln);
+        consume(b1);
+        if (ln >= lb) break;
+        l = ln;
     }
 }
 
@@ -611,7 +783,7 @@ struct Geometry {
     int vec_bytes;  // bytes one lane moves per row
     int lpr_log2;   // log2(lanes that cover one row slice)
     int ytiles;     // column tiles when a row is wider than 64 lanes
-    int n_groups;
+    unsigned lds_fwd, lds_bwd;  // dynamic LDS bytes of the two kernels
     dim3 grid;
 };
 
@@ -635,10 +807,11 @@ Geometry make_geometry(long N, long C, int elem, const void *p0, const void *p1,
     while ((1L << l2) < lanes && l2 < 6) ++l2;
     g.lpr_log2 = l2;
     g.ytiles = (int)((lanes + (1L << l2) - 1) >> l2);
-    g.n_groups = (int)((N + kChunk - 1) / kChunk);
-    const long groups_per_block = kThreads >> l2;
-    long blocks = (g.n_groups + groups_per_block - 1) / groups_per_block;
-    blocks = (blocks + 7) & ~7L;
+    const long tile = (long)(kThreads >> l2) * kChunk;  // sorted positions per workgroup
+    long blocks = (N + tile - 1) / tile;
+    blocks = (blocks + 8 * kXcdSpan - 1) / (8 * kXcdSpan) * (8 * kXcdSpan);
+    g.lds_fwd = (unsigned)((2 * (tile + kMargin) + 1) * sizeof(int));
+    g.lds_bwd = (unsigned)(2 * tile * sizeof(int));
     g.grid = dim3((unsigned)blocks, (unsigned)g.ytiles, 1);
     return g;
 }
@@ -654,16 +827,16 @@ hipError_t launch_fwd_op(int op, const Geometry &geo, hipStream_t st, const void
     dim3 blk(kThreads);
     switch (op) {
         case TXS_SUM:
-            scatter_fwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, 0, st>>>(
-                f, perm, seg, preSum, slot_of, o, arg, s, N, C, U, geo.lpr_log2, geo.n_groups);
+            scatter_fwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, geo.lds_fwd, st>>>(
+                f, perm, seg, slot_of, o, arg, s, N, C, U, geo.lpr_log2);
             break;
         case TXS_MEAN:
-            scatter_fwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, 0, st>>>(
-                f, perm, seg, preSum, slot_of, o, arg, s, N, C, U, geo.lpr_log2, geo.n_groups);
+            scatter_fwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, geo.lds_fwd, st>>>(
+                f, perm, seg, slot_of, o, arg, s, N, C, U, geo.lpr_log2);
             break;
         default:
-            scatter_fwd_kernel<TR, VEC, TXS_MAX><<<geo.grid, blk, 0, st>>>(
-                f, perm, seg, preSum, slot_of, o, arg, s, N, C, U, geo.lpr_log2, geo.n_groups);
+            scatter_fwd_kernel<TR, VEC, TXS_MAX><<<geo.grid, blk, geo.lds_fwd, st>>>(
+                f, perm, seg, slot_of, o, arg, s, N, C, U, geo.lpr_log2);
             break;
     }
     return hipGetLastError();
@@ -726,16 +899,16 @@ hipError_t launch_bwd_op(int op, const Geometry &geo, hipStream_t st, const void
     dim3 blk(kThreads);
     switch (op) {
         case TXS_SUM:
-            scatter_bwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, 0, st>>>(
-                gi, arg, perm, seg, preSum, go, N, C, U, geo.lpr_log2, geo.n_groups);
+            scatter_bwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, geo.lds_bwd, st>>>(
+                gi, arg, perm, seg, preSum, go, N, C, U, geo.lpr_log2);
             break;
         case TXS_MEAN:
-            scatter_bwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, 0, st>>>(
-                gi, arg, perm, seg, preSum, go, N, C, U, geo.lpr_log2, geo.n_groups);
+            scatter_bwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, geo.lds_bwd, st>>>(
+                gi, arg, perm, seg, preSum, go, N, C, U, geo.lpr_log2);
             break;
         default:
-            scatter_bwd_kernel<TR, VEC, TXS_MAX><<<geo.grid, blk, 0, st>>>(
-                gi, arg, perm, seg, preSum, go, N, C, U, geo.lpr_log2, geo.n_groups);
+            scatter_bwd_kernel<TR, VEC, TXS_MAX><<<geo.grid, blk, geo.lds_bwd, st>>>(
+                gi, arg, perm, seg, preSum, go, N, C, U, geo.lpr_log2);
             break;
     }
     return hipGetLastError();

@@ -141,12 +141,16 @@ class ScatterMaxFunction(Function):
         out, arg = _forward(_MAX, feats, data)
         ctx.save_for_backward(arg)
         ctx.mark_non_differentiable(arg)
+        # no zero tensor is made for the gradient slot of the integer output
+        ctx.set_materialize_grads(False)
         ctx.data = data
         return out, arg
 
     @staticmethod
     def backward(ctx, g_out, g_arg):
         # zeros(N, C).scatter_(0, arg, g_out) (scatter_op.py:106-111, as intended)
+        if g_out is None:
+            return None, None
         (arg,) = ctx.saved_tensors
         return _backward(_MAX, g_out, arg, ctx.data), None
 
