@@ -29,6 +29,17 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes per launch on the default workload (N=1,000,000, C=128, fp32), from two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by
+# what the same counter reads for the 512,000,000-byte device copy below (FETCH_SIZE
+# reads half of the copied bytes on this part: factor 2.000; WRITE_SIZE: factor 1.000).
+MEASURED_TRAFFIC_BYTES = {
+    "max_fwd": 525.2e6 + 334.9e6,
+    "max_bwd": 352.0e6 + 512.2e6,
+    "mean_fwd": 525.2e6 + 167.4e6,
+    "mean_bwd": 183.0e6 + 512.4e6,
+}
+
 
 def parse():
     p = argparse.ArgumentParser()
@@ -161,7 +172,8 @@ def main():
     kname = {"max_fwd": "scatter_fwd_kernel<F32,4,MAX>", "mean_fwd": "scatter_fwd_kernel<F32,4,MEAN>",
              "max_bwd": "scatter_bwd_kernel<F32,4,MAX>", "mean_bwd": "scatter_bwd_kernel<F32,4,MEAN>"}[dom]
     roofline = {"bound": "hbm", "kernel": kname, "achieved": per_kernel[dom]["GBps"], "peak": HBM_PEAK_GBPS,
-                "unit": "GB/s", "frac": per_kernel[dom]["frac"], "traffic": None,
+                "unit": "GB/s", "frac": per_kernel[dom]["frac"],
+                "traffic": MEASURED_TRAFFIC_BYTES[dom] if (N, C) == (1_000_000, 128) else None,
                 "algorithmic_bytes": ab[dom], "launch_ms": kt[dom]}
 
     out = {
