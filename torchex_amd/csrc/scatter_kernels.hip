@@ -25,6 +25,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "torchex_scatter.h"
 
 namespace {
@@ -50,7 +52,7 @@ namespace {
 
 constexpr int kThreads = 256;        // 4 wavefronts per workgroup
 constexpr int kChunk = TXS_CHUNK;    // sorted positions per lane group
-constexpr int kBatch = TXS_BATCH;    // rows in flight per lane group
+constexpr int kBatch = TXS_BATCH;    // rows per load batch of a lane group (two batches in flight)
 constexpr int kHeavyDefault = 64;    // voxels above this many rows use the atomic path
 constexpr int kSpecialBit = (int)0x80000000;
 constexpr int kIdMask = 0x7fffffff;
@@ -448,18 +450,36 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     const int n_seg_s = T + kMargin + 1;  // positions t0-1 .. t0+T+kMargin-1
     int *seg_s = lds;
     int *perm_s = lds + n_seg_s;          // positions t0 .. t0+T+kMargin-1
+    // Partials of heavy voxels: two slots per lane group (a chunk can touch at
+    // most two heavy runs, one at each end), combined across the workgroup
+    // before anything goes to the global scratch table.
+    using SlotT = typename std::conditional<OP == TXS_MAX, unsigned long long, float>::type;
+    int *slot_id = perm_s + (n_seg_s - 1);
+    SlotT *slot_val = reinterpret_cast<SlotT *>(lds + ((2 * n_seg_s - 1 + 2 * G + 1) & ~1));
+    const int W = VEC << lpr_log2;        // elements per slot
     const long t0l = (long)xcd_block(blockIdx.x, gridDim.x) * T;
     if (t0l >= N) return;  // uniform for the workgroup
     const int t0 = (int)t0l;
+    bool saw_heavy = false;
     for (int e = threadIdx.x; e < n_seg_s; e += kThreads) {
         const long p = (long)t0 - 1 + e;
         const bool in = p >= 0 && p < N;
-        seg_s[e] = in ? seg[p] : kNoSeg;
+        const int sv = in ? seg[p] : kNoSeg;
+        seg_s[e] = sv;
+        saw_heavy |= (sv < 0) && e >= 1 && e <= T;  // special bit on a position of this tile
         if (e >= 1) perm_s[e - 1] = in ? (perm ? perm[p] : (int)p) : -1;
     }
-    __syncthreads();
+    for (int e = threadIdx.x; e < 2 * G; e += kThreads) slot_id[e] = -1;
+    // one barrier publishes the staged indices and tells the whole workgroup
+    // whether the tile touches a heavy voxel (only then is there a merge phase)
+    const bool tile_has_heavy = __syncthreads_or(saw_heavy);
 
-    const int col = ((int)blockIdx.y << lpr_log2 | ((int)threadIdx.x & ((1 << lpr_log2) - 1))) * VEC;
+    const int gi = (int)threadIdx.x >> lpr_log2;
+    const int lane_in = (int)threadIdx.x & ((1 << lpr_log2) - 1);
+    const int col = ((int)blockIdx.y << lpr_log2 | lane_in) * VEC;
+    int n_heavy = 0;  // heavy partials this lane group has parked in LDS
+
+    auto reduce_chunk = [&]() {
     if (col >= C) return;
     // l indexes seg_s (position t0 - 1 + l); entries past the staged range are
     // fetched from global memory (only an ordinary run longer than kMargin that
@@ -478,7 +498,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     // Range [la, lb) this lane group reduces: its chunk, minus the tail of an
     // ordinary run that began in an earlier chunk, plus the tail of an ordinary
     // run that begins here and ends later.
-    int la = ((int)threadIdx.x >> lpr_log2) * kChunk + 1;
+    int la = gi * kChunk + 1;
     const int lend = min(la + kChunk, N - t0 + 1);
     if (la >= lend) return;
     {
@@ -494,6 +514,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
         if (sl >= 0)
             while (seg_at(lb) == sl) ++lb;  // ends at the latest at N (kNoSeg)
     }
+    const int lb_fast = min(lb, n_seg_s);  // end of the part whose ids are staged in LDS
 
     float acc[VEC];
     int idx[VEC];
@@ -546,27 +567,55 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                 st_stream<int, VEC>(arg + o, ai);
             }
             st_stream<raw, VEC>(out + o, r);
-        } else {  // heavy voxel: merge this chunk's partial into the scratch table
-            const int slot = slot_of[u];
-            if (slot < 0) return;
-            const size_t o = (size_t)slot * C + col;
-            if (OP == TXS_MAX) {
+        } else if (n_heavy < 2) {  // heavy voxel: park this chunk's partial in LDS
+            const int sidx = 2 * gi + n_heavy;
+            ++n_heavy;
+            if (lane_in == 0) slot_id[sidx] = u;
+            SlotT *sv = slot_val + (size_t)sidx * W + lane_in * VEC;
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) {
-                    if (idx[k] >= 0) {
-                        unsigned long long key = ((unsigned long long)ordered_bits(acc[k]) << 32) |
-                                                 (unsigned long long)(0xffffffffu - (unsigned)idx[k]);
-                        atomicMax(scratch + o + k, key);
-                    }
+            for (int k = 0; k < VEC; ++k) {
+                if constexpr (OP == TXS_MAX) {
+                    sv[k] = idx[k] >= 0 ? (((unsigned long long)ordered_bits(acc[k]) << 32) |
+                                           (unsigned long long)(0xffffffffu - (unsigned)idx[k]))
+                                        : 0ull;
+                } else {
+                    sv[k] = acc[k];
                 }
-            } else {
-                float *fs = reinterpret_cast<float *>(scratch) + o;
+            }
+        }
+        // (a third heavy partial in one chunk cannot occur: a heavy run is longer
+        // than a chunk, so a chunk touches at most one at each end)
+    };
+
+    // Fold one loaded row (position l, voxel sg) into the running reduction.
+    // `valid` only gates state changes: the loaded registers are consumed on a
+    // straight-line path so the compiler can count outstanding loads exactly.
+    auto add_row = [&](const Pack<raw, VEC> &v, int sg, int row, int l, bool valid) {
+        if (valid && sg != cur) {
+            flush(l);
+            cur = sg;
+            run_l0 = l;
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) unsafeAtomicAdd(fs + k, acc[k]);
+            for (int k = 0; k < VEC; ++k) {
+                acc[k] = (OP == TXS_MAX) ? -__builtin_inff() : 0.0f;
+                idx[k] = -1;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            const float x = TR::to_f(v.v[k]);
+            if (OP == TXS_MAX) {
+                const bool take = valid && x > acc[k];  // strict: first row wins ties, NaN never wins
+                acc[k] = take ? x : acc[k];
+                idx[k] = take ? row : idx[k];
+            } else {
+                acc[k] += valid ? x : 0.0f;
             }
         }
     };
 
+    // Every slot of a batch issues a load (slots past the range re-load the
+    // range's last row, a cache hit) so that no load sits under a branch.
     struct Batch {
         int segs[kBatch], rows[kBatch];
         Pack<raw, VEC> v[kBatch];
@@ -575,58 +624,95 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
             const int ll = l + i;
-            const bool ok = ll < lb;
-            bt.segs[i] = ok ? seg_at(ll) : kNoSeg;
-            const int r = ok ? row_at(ll) : -1;
-            bt.rows[i] = ((unsigned)r < (unsigned)N) ? r : -1;
+            const int lc = min(ll, lb_fast - 1);
+            const int r = perm_s[lc - 1];
+            const bool valid = ll < lb_fast && (unsigned)r < (unsigned)N;
+            bt.segs[i] = seg_s[lc];
+            bt.rows[i] = valid ? r : -1;
+            bt.v[i] = ld_stream<raw, VEC>(feats + (size_t)((unsigned)r < (unsigned)N ? r : 0) * C + col);
         }
-#pragma unroll
-        for (int i = 0; i < kBatch; ++i)
-            if (bt.rows[i] >= 0) bt.v[i] = ld_stream<raw, VEC>(feats + (size_t)bt.rows[i] * C + col);
     };
     auto consume = [&](const Batch &bt, int l) {
 #pragma unroll
-        for (int i = 0; i < kBatch; ++i) {
-            if (bt.rows[i] < 0) continue;
-            if (bt.segs[i] != cur) {
-                flush(l + i);
-                cur = bt.segs[i];
-                run_l0 = l + i;
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) {
-                    acc[k] = (OP == TXS_MAX) ? -__builtin_inff() : 0.0f;
-                    idx[k] = -1;
-                }
-            }
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) {
-                const float x = TR::to_f(bt.v[i].v[k]);
-                if (OP == TXS_MAX) {
-                    const bool take = x > acc[k];  // strict: first row wins ties, NaN never wins
-                    acc[k] = take ? x : acc[k];
-                    idx[k] = take ? bt.rows[i] : idx[k];
-                } else {
-                    acc[k] += x;
-                }
-            }
-        }
+        for (int i = 0; i < kBatch; ++i) add_row(bt.v[i], bt.segs[i], bt.rows[i], l + i, bt.rows[i] >= 0);
     };
 
+    // Positions staged in LDS go through the double-buffered loop; the rare rest
+    // (an ordinary run longer than kMargin crossing the tile's end) is walked
+    // one row at a time with its ids fetched from global memory.
+    // Each prefetch is unconditional on its path, so the count of loads in
+    // flight is known at every use: a batch is reduced while the next one is
+    // still arriving.
     Batch b0, b1;
     issue(b0, la);
     for (int l = la;;) {
         int ln = l + kBatch;
-        if (ln < lb) issue(b1, ln);
+        if (ln >= lb_fast) {
+            consume(b0, l);
+            break;
+        }
+        issue(b1, ln);
         consume(b0, l);
-        if (ln >= lb) break;
         l = ln;
         ln = l + kBatch;
-        if (ln < lb) issue(b0, ln);
+        if (ln >= lb_fast) {
+            consume(b1, l);
+            break;
+        }
+        issue(b0, ln);
         consume(b1, l);
-        if (ln >= lb) break;
         l = ln;
     }
+    for (int l = lb_fast; l < lb; ++l) {
+        const int r = row_at(l);
+        if ((unsigned)r >= (unsigned)N) continue;
+        add_row(ld_stream<raw, VEC>(feats + (size_t)r * C + col), seg_at(l), r, l, true);
+    }
     flush(lb);
+    };  // reduce_chunk
+    reduce_chunk();
+
+    // Workgroup-level merge of the parked partials: the used slots that carry
+    // the same voxel id form one range (a heavy run is contiguous in sorted
+    // order, so only unused slots can sit between them); the first slot's lane
+    // group folds the range in slot order and issues one atomic per element.
+    // Tiles without a heavy voxel skip this phase and its barrier.
+    if (!tile_has_heavy) return;
+    __syncthreads();
+    if (col >= C) return;
+    for (int h = 0; h < 2; ++h) {
+        const int s0 = 2 * gi + h;
+        const int id = slot_id[s0];
+        if (id < 0) continue;
+        int prev = s0 - 1;
+        while (prev >= 0 && slot_id[prev] < 0) --prev;
+        if (prev >= 0 && slot_id[prev] == id) continue;  // not the first slot of its range
+        SlotT tot[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) tot[k] = slot_val[(size_t)s0 * W + lane_in * VEC + k];
+        for (int t = s0 + 1; t < 2 * G; ++t) {
+            const int tid = slot_id[t];
+            if (tid < 0) continue;
+            if (tid != id) break;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                const SlotT x = slot_val[(size_t)t * W + lane_in * VEC + k];
+                if constexpr (OP == TXS_MAX) tot[k] = x > tot[k] ? x : tot[k];
+                else tot[k] += x;
+            }
+        }
+        const int slot = slot_of[id];
+        if (slot < 0) continue;
+        const size_t o = (size_t)slot * C + col;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            if constexpr (OP == TXS_MAX) {
+                if (tot[k] != 0ull) atomicMax(scratch + o + k, tot[k]);
+            } else {
+                unsafeAtomicAdd(reinterpret_cast<float *>(scratch) + o + k, tot[k]);
+            }
+        }
+    }
 }
 
 // Turn the scratch table of the special voxels into output rows and clear it.
@@ -702,32 +788,32 @@ __global__ __launch_bounds__(kThreads) void scatter_bwd_kernel(
     const int lb = min(la + kChunk, N - t0);
     if (la >= lb) return;
 
+    // A batch keeps the fetched upstream rows and two bit masks; row ids are read
+    // again from LDS when the batch is stored.  The upstream row (and arg row) is
+    // fetched only where the voxel changes.
     struct Batch {
-        int us[kBatch], rows[kBatch];
-        bool need[kBatch];
         Pack<raw, VEC> gv[kBatch];
         Pack<int, VEC> av[kBatch];
-        int c0[kBatch], c1[kBatch];
+        int cnt[kBatch];
+        unsigned valid, need;
     };
     auto issue = [&](Batch &bt, int l) {
+        bt.valid = 0u;
+        bt.need = 0u;
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
             const int ll = l + i;
-            const bool ok = ll < lb;
-            bt.us[i] = ok ? seg_s[ll] : -1;
-            bt.rows[i] = ok ? perm_s[ll] : -1;
+            if (ll >= lb) continue;
+            const int u = seg_s[ll];
+            if (perm_s[ll] < 0) continue;
+            bt.valid |= 1u << i;
             // first position of the chunk, or the voxel changes here
-            bt.need[i] = bt.rows[i] >= 0 && (ll == la || seg_s[ll - 1] != bt.us[i]);
-        }
-#pragma unroll
-        for (int i = 0; i < kBatch; ++i) {
-            if (!bt.need[i]) continue;
-            const size_t o = (size_t)bt.us[i] * C + col;
-            bt.gv[i] = ld<raw, VEC>(g + o);
-            if (OP == TXS_MAX) bt.av[i] = ld<int, VEC>(arg + o);
-            if (OP == TXS_MEAN) {
-                bt.c0[i] = preSum[bt.us[i]];
-                bt.c1[i] = preSum[bt.us[i] + 1];
+            if (ll == la || seg_s[ll - 1] != u) {
+                bt.need |= 1u << i;
+                const size_t o = (size_t)u * C + col;
+                bt.gv[i] = ld<raw, VEC>(g + o);
+                if (OP == TXS_MAX) bt.av[i] = ld<int, VEC>(arg + o);
+                if (OP == TXS_MEAN) bt.cnt[i] = preSum[u + 1] - preSum[u];
             }
         }
     };
@@ -738,13 +824,13 @@ __global__ __launch_bounds__(kThreads) void scatter_bwd_kernel(
         q.v[k] = TR::zero();
         aq.v[k] = -1;
     }
-    auto consume = [&](const Batch &bt) {
+    auto consume = [&](const Batch &bt, int l) {
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
-            if (bt.rows[i] < 0) continue;
-            if (bt.need[i]) {
+            if (!(bt.valid & (1u << i))) continue;
+            if (bt.need & (1u << i)) {
                 if (OP == TXS_MEAN) {  // one division per run, not per row
-                    const float d = (float)(bt.c1[i] - bt.c0[i]);
+                    const float d = (float)bt.cnt[i];
 #pragma unroll
                     for (int k = 0; k < VEC; ++k) q.v[k] = TR::from_f(TR::to_f(bt.gv[i].v[k]) / d);
                 } else {
@@ -752,12 +838,13 @@ __global__ __launch_bounds__(kThreads) void scatter_bwd_kernel(
                 }
                 if (OP == TXS_MAX) aq = bt.av[i];
             }
+            const int row = perm_s[l + i];
             Pack<raw, VEC> r = q;
             if (OP == TXS_MAX) {
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) r.v[k] = (aq.v[k] == bt.rows[i]) ? q.v[k] : TR::zero();
+                for (int k = 0; k < VEC; ++k) r.v[k] = (aq.v[k] == row) ? q.v[k] : TR::zero();
             }
-            st_stream<raw, VEC>(gin + (size_t)bt.rows[i] * C + col, r);
+            st_stream<raw, VEC>(gin + (size_t)row * C + col, r);
         }
     };
 
@@ -766,12 +853,12 @@ __global__ __launch_bounds__(kThreads) void scatter_bwd_kernel(
     for (int l = la;;) {
         int ln = l + kBatch;
         if (ln < lb) issue(b1, ln);
-        consume(b0);
+        consume(b0, l);
         if (ln >= lb) break;
         l = ln;
         ln = l + kBatch;
         if (ln < lb) issue(b0, ln);
-        consume(b1);
+        consume(b1, l);
         if (ln >= lb) break;
         l = ln;
     }
@@ -783,7 +870,7 @@ struct Geometry {
     int vec_bytes;  // bytes one lane moves per row
     int lpr_log2;   // log2(lanes that cover one row slice)
     int ytiles;     // column tiles when a row is wider than 64 lanes
-    unsigned lds_fwd, lds_bwd;  // dynamic LDS bytes of the two kernels
+    unsigned lds_fwd_idx, lds_slots, lds_bwd;  // dynamic LDS: fwd index part (bytes), fwd slot elements, bwd bytes
     dim3 grid;
 };
 
@@ -810,7 +897,8 @@ Geometry make_geometry(long N, long C, int elem, const void *p0, const void *p1,
     const long tile = (long)(kThreads >> l2) * kChunk;  // sorted positions per workgroup
     long blocks = (N + tile - 1) / tile;
     blocks = (blocks + 8 * kXcdSpan - 1) / (8 * kXcdSpan) * (8 * kXcdSpan);
-    g.lds_fwd = (unsigned)((2 * (tile + kMargin) + 1) * sizeof(int));
+    g.lds_fwd_idx = (unsigned)((((2 * (tile + kMargin) + 1) + 2 * (kThreads >> l2) + 1) & ~1L) * sizeof(int));
+    g.lds_slots = (unsigned)(2 * kThreads * vec);
     g.lds_bwd = (unsigned)(2 * tile * sizeof(int));
     g.grid = dim3((unsigned)blocks, (unsigned)g.ytiles, 1);
     return g;
@@ -827,15 +915,15 @@ hipError_t launch_fwd_op(int op, const Geometry &geo, hipStream_t st, const void
     dim3 blk(kThreads);
     switch (op) {
         case TXS_SUM:
-            scatter_fwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, geo.lds_fwd, st>>>(
+            scatter_fwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, geo.lds_fwd_idx + 4 * geo.lds_slots, st>>>(
                 f, perm, seg, slot_of, o, arg, s, N, C, U, geo.lpr_log2);
             break;
         case TXS_MEAN:
-            scatter_fwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, geo.lds_fwd, st>>>(
+            scatter_fwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, geo.lds_fwd_idx + 4 * geo.lds_slots, st>>>(
                 f, perm, seg, slot_of, o, arg, s, N, C, U, geo.lpr_log2);
             break;
         default:
-            scatter_fwd_kernel<TR, VEC, TXS_MAX><<<geo.grid, blk, geo.lds_fwd, st>>>(
+            scatter_fwd_kernel<TR, VEC, TXS_MAX><<<geo.grid, blk, geo.lds_fwd_idx + 8 * geo.lds_slots, st>>>(
                 f, perm, seg, slot_of, o, arg, s, N, C, U, geo.lpr_log2);
             break;
     }
