@@ -55,6 +55,7 @@ enum {
     TXS_STAT_MAX_CNT = 2,      /* largest voxel population */
     TXS_STAT_NUM_SPECIAL = 3,  /* number of special voxels (heavy or empty) */
     TXS_STAT_NUM_EMPTY = 4,    /* number of voxels with zero rows */
+    TXS_STAT_COUNT_MISMATCH = 5, /* 1 if the caller's unq_cnts is not the histogram of unq_inv */
     TXS_STATS_LEN = 8
 };
 
@@ -79,39 +80,47 @@ int txs_chunk_rows(void);
 int txs_get_presum(const int32_t *unq_inv, int32_t *preSum, int64_t num_total,
                    int64_t num_presum, void *stream);
 
-/* Exact histogram of unq_inv plus order / range checks.  Extends
- * ScatterData.__init__ (scatter_op.py:13-21) to unsorted input.
- * counts [U] and stats [TXS_STATS_LEN] are zeroed by the call. */
-int txs_plan_count(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
-                   int32_t *counts, int32_t *stats, void *stream);
+/* Order and range flags of unq_inv: sets stats[UNSORTED] / stats[OUT_OF_RANGE].
+ * First step of what ScatterData.__init__ (scatter_op.py:13-21) does, extended
+ * to unsorted input.  stats [TXS_STATS_LEN] must be zero-filled by the caller;
+ * the plan calls below accumulate into it and nothing is read back by the
+ * library, so the whole plan needs one host synchronisation (to read stats). */
+int txs_plan_check(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, int32_t *stats,
+                   void *stream);
 
-/* preSum = [0, cumsum(counts)], the special-voxel table and max_cnt.
- * scan_ws: int32 workspace of txs_scan_workspace_len(num_unq) entries.
- * heavy_ids must hold num_unq entries (only the first NUM_SPECIAL are used).
- * For sorted input preSum equals what txs_get_presum produces. */
-int txs_plan_offsets(const int32_t *counts, int64_t num_unq, int32_t heavy_threshold,
-                     int32_t *preSum, int32_t *slot_of, int32_t *heavy_ids, int32_t *stats,
-                     int32_t *scan_ws, void *stream);
-int64_t txs_scan_workspace_len(int64_t n);
-
-/* Stable sort of row ids by voxel id (LSD radix, 3-kernel passes, no
- * inter-block spinning): fills perm and seg.  sort_ws: int32 workspace of
+/* Sorted keys and the stable permutation: keys[j] = voxel id at sorted position
+ * j, perm[j] = its row (ascending rows inside a voxel).  LSD radix sort, three
+ * kernels per pass, no inter-block spinning.  When stats[UNSORTED] is 0 (read
+ * on the device) the passes return at once, keys becomes a copy of unq_inv and
+ * perm is left unwritten (position == row).  sort_ws: int32 workspace of
  * txs_sort_workspace_len(num_total, num_unq) entries. */
-int txs_plan_sort(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
-                  const int32_t *slot_of, int32_t *perm, int32_t *seg, int32_t *sort_ws,
-                  void *stream);
+int txs_plan_sort(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, const int32_t *stats,
+                  int32_t *perm, int32_t *keys, int32_t *sort_ws, void *stream);
 int64_t txs_sort_workspace_len(int64_t num_total, int64_t num_unq);
 
-/* seg for input that is already sorted (perm == NULL): seg[j] = unq_inv[j]
- * with the special bit from slot_of. */
-int txs_plan_seg_sorted(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
-                        const int32_t *slot_of, int32_t *seg, void *stream);
+/* CSR offsets from sorted keys: preSum[u] = first sorted position with key >= u,
+ * preSum[num_unq] = num_total (no atomics, no scan).  On sorted input this is
+ * what txs_get_presum / the reference's getPreSum produce, with empty voxels
+ * handled too. */
+int txs_plan_presum(const int32_t *sorted_keys, int64_t num_total, int64_t num_unq,
+                    int32_t *preSum, void *stream);
 
-/* counts from CSR offsets, for callers that hold only preSum (the reference's
- * scatter_ext.sum / scatter_ext.max argument lists, scatter.cpp:20-53), and
- * seg by binary search of each position in preSum. */
-int txs_counts_from_presum(const int32_t *preSum, int64_t num_unq, int32_t *counts,
-                           int32_t *stats, void *stream);
+/* Table of special voxels (heavy or empty) from CSR offsets, stats[MAX_CNT],
+ * stats[NUM_SPECIAL], stats[NUM_EMPTY]; when unq_cnts (int64 [num_unq], as
+ * torch.unique returns it) is given, stats[COUNT_MISMATCH] is set if it is not
+ * the histogram of unq_inv (the consistency check of scatter_op.py:19).
+ * heavy_ids must hold num_unq entries (the first NUM_SPECIAL are used). */
+int txs_plan_special(const int32_t *preSum, int64_t num_unq, int32_t heavy_threshold,
+                     const int64_t *unq_cnts, int32_t *slot_of, int32_t *heavy_ids, int32_t *stats,
+                     void *stream);
+
+/* In place: sorted keys -> seg (sets bit 31 on positions of special voxels). */
+int txs_plan_seg_flag(int32_t *keys_to_seg, int64_t num_total, int64_t num_unq,
+                      const int32_t *slot_of, void *stream);
+
+/* seg by binary search of each position in preSum, for callers that hold only
+ * CSR offsets of already grouped rows (the reference's scatter_ext.sum /
+ * scatter_ext.max argument lists, scatter.cpp:20-53). */
 int txs_plan_seg_from_presum(const int32_t *preSum, int64_t num_total, int64_t num_unq,
                              const int32_t *slot_of, int32_t *seg, void *stream);
 

@@ -71,56 +71,48 @@ std::vector<int64_t> read_stats(const Tensor &stats) {
     return v;
 }
 
-// counts -> preSum, special table, stats (shared tail of both plan builders)
-struct Offsets {
-    Tensor preSum, slot_of, heavy_ids;
-};
-
-Offsets plan_offsets(const Tensor &counts, int64_t U, int64_t heavy_threshold, Tensor &stats) {
-    Offsets o;
-    o.preSum = empty_i32(U + 1, counts);
-    o.slot_of = empty_i32(U, counts);
-    o.heavy_ids = empty_i32(U, counts);
-    Tensor ws = empty_i32(txs_scan_workspace_len(U), counts);
-    check_status(txs_plan_offsets(i32p(counts), U, (int32_t)heavy_threshold, i32w(o.preSum),
-                                  i32w(o.slot_of), i32w(o.heavy_ids), i32w(stats), i32w(ws),
-                                  cur_stream(counts)),
-                 "plan_offsets");
-    return o;
-}
-
 // ScatterData index preparation for an unq_inv in any order
-// (extends torchex/operator_py/scatter_op.py:13-21).
+// (extends torchex/operator_py/scatter_op.py:13-21).  Everything is queued on
+// the current stream; the only host synchronisation is the read of `stats`.
 // returns (preSum, perm | None, seg, slot_of, heavy_ids, stats)
 std::tuple<Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>> build_plan(
-    const Tensor &unq_inv, int64_t num_unq, int64_t heavy_threshold) {
+    const Tensor &unq_inv, int64_t num_unq, int64_t heavy_threshold, const OptTensor &unq_cnts) {
     check_i32(unq_inv, "unq_inv");
     TORCH_CHECK(unq_inv.dim() == 1, "unq_inv must be 1-D");
     TORCH_CHECK(num_unq >= 0, "num_unq must be non-negative");
+    const int64_t *cnts = nullptr;
+    if (unq_cnts.has_value()) {
+        check_dev(*unq_cnts, "unq_cnts");
+        TORCH_CHECK(unq_cnts->scalar_type() == at::kLong && unq_cnts->numel() == num_unq,
+                    "unq_cnts must be int64 with num_unq entries");
+        cnts = num_unq ? unq_cnts->data_ptr<int64_t>() : nullptr;
+    }
     c10::hip::HIPGuardMasqueradingAsCUDA guard(unq_inv.device());
     const int64_t N = unq_inv.numel(), U = num_unq;
-    Tensor counts = empty_i32(U, unq_inv);
-    Tensor stats = empty_i32(TXS_STATS_LEN, unq_inv);
     void *st = cur_stream(unq_inv);
-    check_status(txs_plan_count(i32p(unq_inv), N, U, i32w(counts), i32w(stats), st), "plan_count");
-    Offsets o = plan_offsets(counts, U, heavy_threshold, stats);
-    std::vector<int64_t> hs = read_stats(stats);
-    TORCH_CHECK(hs[TXS_STAT_OUT_OF_RANGE] == 0, "unq_inv holds ids outside [0, num_unq=", U, ")");
+    Tensor stats = at::zeros({TXS_STATS_LEN}, unq_inv.options());
     Tensor seg = empty_i32(N, unq_inv);
-    OptTensor perm;
-    if (hs[TXS_STAT_UNSORTED]) {
-        Tensor p = empty_i32(N, unq_inv);
-        Tensor ws = empty_i32(txs_sort_workspace_len(N, U), unq_inv);
-        check_status(txs_plan_sort(i32p(unq_inv), N, U, i32p(o.slot_of), i32w(p), i32w(seg),
-                                   i32w(ws), st),
+    Tensor perm = empty_i32(N, unq_inv);
+    Tensor ws = empty_i32(txs_sort_workspace_len(N, U), unq_inv);
+    Tensor preSum = empty_i32(U + 1, unq_inv);
+    Tensor slot_of = empty_i32(U, unq_inv);
+    Tensor heavy_all = empty_i32(U, unq_inv);
+    check_status(txs_plan_check(i32p(unq_inv), N, U, i32w(stats), st), "plan_check");
+    if (U > 0)
+        check_status(txs_plan_sort(i32p(unq_inv), N, U, i32p(stats), i32w(perm), i32w(seg), i32w(ws), st),
                      "plan_sort");
-        perm = p;
-    } else {
-        check_status(txs_plan_seg_sorted(i32p(unq_inv), N, U, i32p(o.slot_of), i32w(seg), st),
-                     "plan_seg_sorted");
-    }
-    Tensor heavy_ids = o.heavy_ids.narrow(0, 0, hs[TXS_STAT_NUM_SPECIAL]).contiguous();
-    return {o.preSum, perm, seg, o.slot_of, heavy_ids, hs};
+    check_status(txs_plan_presum(i32p(seg), U > 0 ? N : 0, U, i32w(preSum), st), "plan_presum");
+    check_status(txs_plan_special(i32p(preSum), U, (int32_t)heavy_threshold, cnts, i32w(slot_of),
+                                  i32w(heavy_all), i32w(stats), st),
+                 "plan_special");
+    check_status(txs_plan_seg_flag(i32w(seg), U > 0 ? N : 0, U, i32p(slot_of), st), "plan_seg_flag");
+    std::vector<int64_t> hs = read_stats(stats);
+    TORCH_CHECK(hs[TXS_STAT_OUT_OF_RANGE] == 0 && (U > 0 || N == 0),
+                "unq_inv holds ids outside [0, num_unq=", U, ")");
+    OptTensor perm_out;
+    if (hs[TXS_STAT_UNSORTED]) perm_out = perm;
+    Tensor heavy_ids = heavy_all.narrow(0, 0, hs[TXS_STAT_NUM_SPECIAL]).contiguous();
+    return {preSum, perm_out, seg, slot_of, heavy_ids, hs};
 }
 
 // Plan for callers that hold only CSR offsets of already grouped rows.
@@ -132,17 +124,19 @@ std::tuple<Tensor, Tensor, Tensor, std::vector<int64_t>> plan_from_presum(
     c10::hip::HIPGuardMasqueradingAsCUDA guard(preSum.device());
     const int64_t U = preSum.numel() - 1, N = num_total;
     void *st = cur_stream(preSum);
-    Tensor counts = empty_i32(U, preSum);
-    Tensor stats = empty_i32(TXS_STATS_LEN, preSum);
-    check_status(txs_counts_from_presum(i32p(preSum), U, i32w(counts), i32w(stats), st),
-                 "counts_from_presum");
-    Offsets o = plan_offsets(counts, U, heavy_threshold, stats);
-    std::vector<int64_t> hs = read_stats(stats);
+    Tensor stats = at::zeros({TXS_STATS_LEN}, preSum.options());
+    Tensor slot_of = empty_i32(U, preSum);
+    Tensor heavy_all = empty_i32(U, preSum);
+    check_status(txs_plan_special(i32p(preSum), U, (int32_t)heavy_threshold, nullptr, i32w(slot_of),
+                                  i32w(heavy_all), i32w(stats), st),
+                 "plan_special");
     Tensor seg = empty_i32(N, preSum);
-    check_status(txs_plan_seg_from_presum(i32p(preSum), N, U, i32p(o.slot_of), i32w(seg), st),
-                 "plan_seg_from_presum");
-    Tensor heavy_ids = o.heavy_ids.narrow(0, 0, hs[TXS_STAT_NUM_SPECIAL]).contiguous();
-    return {seg, o.slot_of, heavy_ids, hs};
+    if (U > 0)
+        check_status(txs_plan_seg_from_presum(i32p(preSum), N, U, i32p(slot_of), i32w(seg), st),
+                     "plan_seg_from_presum");
+    std::vector<int64_t> hs = read_stats(stats);
+    Tensor heavy_ids = heavy_all.narrow(0, 0, hs[TXS_STAT_NUM_SPECIAL]).contiguous();
+    return {seg, slot_of, heavy_ids, hs};
 }
 
 Tensor make_scratch(int64_t num_special, int64_t C, const Tensor &like) {
@@ -271,7 +265,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("sum", &sum_ref, "scatter_sum over CSR offsets, in place (HIP)");
     m.def("max", &max_ref, "scatter_max with arg over CSR offsets, in place (HIP)");
     m.def("getPreSum", &get_presum_ref, "CSR offsets from a sorted unq_inv (HIP)");
-    m.def("build_plan", &build_plan, "index preparation for unq_inv in any order");
+    m.def("build_plan", &build_plan, "build_plan(unq_inv, num_unq, heavy_threshold, unq_cnts|None)");
     m.def("plan_from_presum", &plan_from_presum, "index preparation from CSR offsets");
     m.def("make_scratch", &make_scratch, "zeroed scratch table for the special voxels");
     m.def("forward", &forward, "forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch)");

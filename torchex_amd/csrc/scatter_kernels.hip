@@ -179,23 +179,37 @@ __global__ void get_presum_kernel(const int *__restrict__ inv, int *__restrict__
     if (boundary && slot >= 0 && slot < num_presum) preSum[slot] = (int)(i + 1);
 }
 
-__global__ void plan_count_kernel(const int *__restrict__ inv, long n, int U,
-                                  int *__restrict__ counts, int *__restrict__ stats) {
+// Order and range flags of unq_inv (no histogram: counts come from the run
+// boundaries of the sorted ids, which needs no atomics).
+__global__ void plan_check_kernel(const int *__restrict__ inv, long n, int U,
+                                  int *__restrict__ stats) {
     long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    int v = inv[i];
-    if ((unsigned)v >= (unsigned)U) {
-        stats[TXS_STAT_OUT_OF_RANGE] = 1;
-        return;
-    }
-    atomicAdd(&counts[v], 1);
+    const int v = inv[i];
+    if ((unsigned)v >= (unsigned)U) stats[TXS_STAT_OUT_OF_RANGE] = 1;
     if (i + 1 < n && inv[i + 1] < v) stats[TXS_STAT_UNSORTED] = 1;
 }
 
-__global__ void counts_from_presum_kernel(const int *__restrict__ preSum, int U,
-                                          int *__restrict__ counts) {
-    int u = blockIdx.x * blockDim.x + threadIdx.x;
-    if (u < U) counts[u] = preSum[u + 1] - preSum[u];
+// ids that are already sorted are their own sorted keys
+__global__ void copy_if_sorted_kernel(const int *__restrict__ inv, long n,
+                                      const int *__restrict__ stats, int *__restrict__ keys) {
+    if (stats[TXS_STAT_UNSORTED] != 0) return;
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) keys[i] = inv[i];
+}
+
+// CSR offsets from sorted keys: preSum[u] = first position whose key is >= u.
+// Thread j owns the boundary in front of position j and fills the offsets of
+// every id in (key[j-1], key[j]] (more than one only across empty voxels).
+__global__ void presum_from_sorted_kernel(const int *__restrict__ keys, long n, int U,
+                                          int *__restrict__ preSum) {
+    long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j > n) return;
+    long lo = (j == 0) ? -1 : (long)(keys[j - 1] & kIdMask);
+    long hi = (j == n) ? (long)U : (long)(keys[j] & kIdMask);
+    if (hi > U) hi = U;
+    for (long u = lo + 1; u <= hi; ++u)
+        if (u >= 0) preSum[u] = (int)j;
 }
 
 // ------------------------------------------------------------ exclusive scan --
@@ -298,16 +312,32 @@ hipError_t exclusive_scan(const int *in, long n_in, int *out, long n_out, int *w
     return hipGetLastError();
 }
 
-// special-voxel table and max_cnt
-__global__ void plan_special_kernel(const int *__restrict__ counts, int U, int heavy_threshold,
+__device__ __forceinline__ int wave_max_i32(int x) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) x = max(x, __shfl_xor(x, d, 64));
+    return x;
+}
+
+// Special-voxel table, max_cnt, and the check of the caller's counts against
+// the histogram.  One atomic per wavefront for the statistics.
+__global__ void plan_special_kernel(const int *__restrict__ preSum, int U, int heavy_threshold,
+                                    const long long *__restrict__ unq_cnts,
                                     int *__restrict__ slot_of, int *__restrict__ heavy_ids,
                                     int *__restrict__ stats) {
-    int u = blockIdx.x * blockDim.x + threadIdx.x;
-    if (u >= U) return;
-    int c = counts[u];
-    atomicMax(&stats[TXS_STAT_MAX_CNT], c);
+    const int u = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool in = u < U;
+    const int c = in ? preSum[u + 1] - preSum[u] : 0;
+    const int wmax = wave_max_i32(c);
+    const int n_empty = __popcll(__ballot(in && c == 0));
+    const bool mismatch = in && unq_cnts && unq_cnts[u] != (long long)c;
+    const bool any_mismatch = __ballot(mismatch) != 0ull;
+    if ((threadIdx.x & 63) == 0) {
+        if (wmax > 0) atomicMax(&stats[TXS_STAT_MAX_CNT], wmax);
+        if (n_empty) atomicAdd(&stats[TXS_STAT_NUM_EMPTY], n_empty);
+        if (any_mismatch) stats[TXS_STAT_COUNT_MISMATCH] = 1;
+    }
+    if (!in) return;
     int slot = -1;
-    if (c == 0) atomicAdd(&stats[TXS_STAT_NUM_EMPTY], 1);
     if (c > heavy_threshold || c == 0) {
         slot = atomicAdd(&stats[TXS_STAT_NUM_SPECIAL], 1);
         if (slot < U) heavy_ids[slot] = u;
@@ -327,8 +357,10 @@ constexpr int kSortWaveSpan = 64 * kSortItems;    // 512 consecutive keys per wa
 
 __global__ __launch_bounds__(kThreads) void sort_hist_kernel(const int *__restrict__ keys, long n,
                                                              int shift, int rbits,
-                                                             int *__restrict__ hist, int n_tiles) {
+                                                             int *__restrict__ hist, int n_tiles,
+                                                             const int *__restrict__ stats) {
     __shared__ int h[256];
+    if (stats[TXS_STAT_UNSORTED] == 0) return;  // nothing to sort
     const int R = 1 << rbits;
     h[threadIdx.x] = 0;
     __syncthreads();
@@ -345,8 +377,9 @@ __global__ __launch_bounds__(kThreads) void sort_hist_kernel(const int *__restri
 __global__ __launch_bounds__(kThreads) void sort_scatter_kernel(
     const int *__restrict__ keys_in, const int *__restrict__ vals_in, int *__restrict__ keys_out,
     int *__restrict__ vals_out, long n, int shift, int rbits, const int *__restrict__ hist_scanned,
-    int n_tiles) {
+    int n_tiles, const int *__restrict__ stats) {
     __shared__ int wcount[kSortWaves][256];
+    if (stats[TXS_STAT_UNSORTED] == 0) return;  // nothing to sort
     __shared__ int woff[kSortWaves][256];
     const int R = 1 << rbits;
     const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -401,8 +434,8 @@ __global__ __launch_bounds__(kThreads) void sort_scatter_kernel(
 }
 
 // seg[j] = id | special bit
-__global__ void seg_flag_kernel(const int *__restrict__ ids, long n, int U,
-                                const int *__restrict__ slot_of, int *__restrict__ seg) {
+__global__ void seg_flag_kernel(const int *ids, long n, int U, const int *__restrict__ slot_of,
+                                int *seg) {
     long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (j >= n) return;
     int u = ids[j] & kIdMask;
@@ -1039,7 +1072,7 @@ int radix_bits(int64_t U) {
 
 extern "C" {
 
-int txs_abi_version(void) { return 1; }
+int txs_abi_version(void) { return 2; }
 
 const char *txs_status_string(int status) {
     switch (status) {
@@ -1064,34 +1097,13 @@ int txs_get_presum(const int32_t *unq_inv, int32_t *preSum, int64_t num_total, i
     return status_of(hipGetLastError());
 }
 
-int txs_plan_count(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, int32_t *counts,
-                   int32_t *stats, void *stream) {
+int txs_plan_check(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, int32_t *stats,
+                   void *stream) {
     if (!fits_i32(num_total) || !fits_i32(num_unq) || !stats) return TXS_ERR_INVALID_ARG;
-    if ((num_total > 0 && !unq_inv) || (num_unq > 0 && !counts)) return TXS_ERR_INVALID_ARG;
-    hipStream_t st = (hipStream_t)stream;
-    fill_i32_kernel<<<dim3(1), dim3(64), 0, st>>>(stats, TXS_STATS_LEN, 0);
-    if (num_unq > 0)
-        fill_i32_kernel<<<dim3(blocks_for(num_unq)), dim3(kThreads), 0, st>>>(counts, num_unq, 0);
-    if (num_total > 0)
-        plan_count_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, st>>>(
-            unq_inv, num_total, (int)num_unq, counts, stats);
-    return status_of(hipGetLastError());
-}
-
-int64_t txs_scan_workspace_len(int64_t n) { return scan_tiles(n + 1) + 1; }
-
-int txs_plan_offsets(const int32_t *counts, int64_t num_unq, int32_t heavy_threshold,
-                     int32_t *preSum, int32_t *slot_of, int32_t *heavy_ids, int32_t *stats,
-                     int32_t *scan_ws, void *stream) {
-    if (!fits_i32(num_unq) || !preSum || !stats || !scan_ws || heavy_threshold < kChunk)
-        return TXS_ERR_INVALID_ARG;
-    if (num_unq > 0 && (!counts || !slot_of || !heavy_ids)) return TXS_ERR_INVALID_ARG;
-    hipStream_t st = (hipStream_t)stream;
-    hipError_t e = exclusive_scan(counts, num_unq, preSum, num_unq + 1, scan_ws, st);
-    if (e != hipSuccess) return TXS_ERR_LAUNCH;
-    if (num_unq > 0)
-        plan_special_kernel<<<dim3(blocks_for(num_unq)), dim3(kThreads), 0, st>>>(
-            counts, (int)num_unq, heavy_threshold, slot_of, heavy_ids, stats);
+    if (num_total == 0) return TXS_OK;
+    if (!unq_inv) return TXS_ERR_INVALID_ARG;
+    plan_check_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+        unq_inv, num_total, (int)num_unq, stats);
     return status_of(hipGetLastError());
 }
 
@@ -1100,15 +1112,14 @@ int64_t txs_sort_workspace_len(int64_t num_total, int64_t num_unq) {
     const int64_t hist = 256 * (tiles > 0 ? tiles : 1);
     (void)num_unq;
     // two ping-pong arrays, the digit-major histogram, and the scan workspace
-    return 2 * num_total + hist + txs_scan_workspace_len(hist) + 16;
+    return 2 * num_total + hist + scan_tiles(hist + 1) + 17;
 }
 
-int txs_plan_sort(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
-                  const int32_t *slot_of, int32_t *perm, int32_t *seg, int32_t *sort_ws,
-                  void *stream) {
+int txs_plan_sort(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, const int32_t *stats,
+                  int32_t *perm, int32_t *keys, int32_t *sort_ws, void *stream) {
     if (!fits_i32(num_total) || !fits_i32(num_unq)) return TXS_ERR_INVALID_ARG;
     if (num_total == 0) return TXS_OK;
-    if (!unq_inv || !slot_of || !perm || !seg || !sort_ws || num_unq <= 0) return TXS_ERR_INVALID_ARG;
+    if (!unq_inv || !stats || !perm || !keys || !sort_ws || num_unq <= 0) return TXS_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const long n = num_total;
     const int n_tiles = (int)((n + kSortTile - 1) / kSortTile);
@@ -1118,6 +1129,7 @@ int txs_plan_sort(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
     int *hist = sort_ws + 2 * n;
     int *scan_ws = hist + hist_len;
 
+    copy_if_sorted_kernel<<<dim3(blocks_for(n)), dim3(kThreads), 0, st>>>(unq_inv, n, stats, keys);
     const int bits = radix_bits(num_unq);
     const int passes = (bits + 7) / 8;
     const int rbits = (bits + passes - 1) / passes;
@@ -1125,41 +1137,48 @@ int txs_plan_sort(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
     const int *vin = nullptr;  // identity
     for (int p = 0; p < passes; ++p) {
         const bool to_final = ((passes - 1 - p) % 2) == 0;
-        int *kout = to_final ? seg : tmp_keys;
+        int *kout = to_final ? keys : tmp_keys;
         int *vout = to_final ? perm : tmp_vals;
         const int shift = p * rbits;
-        sort_hist_kernel<<<dim3(n_tiles), dim3(kThreads), 0, st>>>(kin, n, shift, rbits, hist, n_tiles);
+        sort_hist_kernel<<<dim3(n_tiles), dim3(kThreads), 0, st>>>(kin, n, shift, rbits, hist, n_tiles,
+                                                                  stats);
         const long used = (1L << rbits) * n_tiles;
         if (exclusive_scan(hist, used, hist, used, scan_ws, st) != hipSuccess) return TXS_ERR_LAUNCH;
         sort_scatter_kernel<<<dim3(n_tiles), dim3(kThreads), 0, st>>>(kin, vin, kout, vout, n, shift,
-                                                                     rbits, hist, n_tiles);
+                                                                     rbits, hist, n_tiles, stats);
         kin = kout;
         vin = vout;
     }
-    seg_flag_kernel<<<dim3(blocks_for(n)), dim3(kThreads), 0, st>>>(seg, n, (int)num_unq, slot_of, seg);
     return status_of(hipGetLastError());
 }
 
-int txs_plan_seg_sorted(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
-                        const int32_t *slot_of, int32_t *seg, void *stream) {
+int txs_plan_presum(const int32_t *sorted_keys, int64_t num_total, int64_t num_unq, int32_t *preSum,
+                    void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_unq) || !preSum) return TXS_ERR_INVALID_ARG;
+    if (num_total > 0 && !sorted_keys) return TXS_ERR_INVALID_ARG;
+    presum_from_sorted_kernel<<<dim3(blocks_for(num_total + 1)), dim3(kThreads), 0,
+                                (hipStream_t)stream>>>(sorted_keys, num_total, (int)num_unq, preSum);
+    return status_of(hipGetLastError());
+}
+
+int txs_plan_special(const int32_t *preSum, int64_t num_unq, int32_t heavy_threshold,
+                     const int64_t *unq_cnts, int32_t *slot_of, int32_t *heavy_ids, int32_t *stats,
+                     void *stream) {
+    if (!fits_i32(num_unq) || !preSum || !stats || heavy_threshold < kChunk) return TXS_ERR_INVALID_ARG;
+    if (num_unq == 0) return TXS_OK;
+    if (!slot_of || !heavy_ids) return TXS_ERR_INVALID_ARG;
+    plan_special_kernel<<<dim3(blocks_for(num_unq)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+        preSum, (int)num_unq, heavy_threshold, (const long long *)unq_cnts, slot_of, heavy_ids, stats);
+    return status_of(hipGetLastError());
+}
+
+int txs_plan_seg_flag(int32_t *keys_to_seg, int64_t num_total, int64_t num_unq,
+                      const int32_t *slot_of, void *stream) {
     if (!fits_i32(num_total) || !fits_i32(num_unq)) return TXS_ERR_INVALID_ARG;
     if (num_total == 0) return TXS_OK;
-    if (!unq_inv || !slot_of || !seg) return TXS_ERR_INVALID_ARG;
+    if (!keys_to_seg || !slot_of) return TXS_ERR_INVALID_ARG;
     seg_flag_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
-        unq_inv, num_total, (int)num_unq, slot_of, seg);
-    return status_of(hipGetLastError());
-}
-
-int txs_counts_from_presum(const int32_t *preSum, int64_t num_unq, int32_t *counts, int32_t *stats,
-                           void *stream) {
-    if (!fits_i32(num_unq) || !preSum || !stats) return TXS_ERR_INVALID_ARG;
-    hipStream_t st = (hipStream_t)stream;
-    fill_i32_kernel<<<dim3(1), dim3(64), 0, st>>>(stats, TXS_STATS_LEN, 0);
-    if (num_unq > 0) {
-        if (!counts) return TXS_ERR_INVALID_ARG;
-        counts_from_presum_kernel<<<dim3(blocks_for(num_unq)), dim3(kThreads), 0, st>>>(
-            preSum, (int)num_unq, counts);
-    }
+        keys_to_seg, num_total, (int)num_unq, slot_of, keys_to_seg);
     return status_of(hipGetLastError());
 }
 

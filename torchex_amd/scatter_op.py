@@ -50,13 +50,12 @@ class ScatterData:
         self.heavy_threshold = int(heavy_threshold)
         flat = self.unq_inv.reshape(-1).contiguous()
         num_unq = self.unq_cnts.shape[0]
+        cnts64 = self.unq_cnts.reshape(-1).long().contiguous()
         (self.preSum, self.perm, self.seg, self.slot_of, self.heavy_ids,
-         stats) = scatter_ext.build_plan(flat, num_unq, self.heavy_threshold)
+         stats) = scatter_ext.build_plan(flat, num_unq, self.heavy_threshold, cnts64)
         # same consistency check as the reference (scatter_op.py:19), made on
         # the recomputed histogram so that a stale unq_cnts is caught too
-        counts = self.preSum[1:] - self.preSum[:-1]
-        assert torch.equal(counts, self.unq_cnts.reshape(-1).to(counts.dtype)), \
-            "unq_cnts is not the histogram of unq_inv"
+        assert stats[5] == 0, "unq_cnts is not the histogram of unq_inv"
         self.num_total = flat.shape[0]
         self.is_sorted = self.perm is None
         self.max_cnt = int(stats[2])
