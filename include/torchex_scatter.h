@@ -46,7 +46,7 @@ extern "C" {
 
 enum { TXS_OK = 0, TXS_ERR_INVALID_ARG = 1, TXS_ERR_LAUNCH = 2, TXS_ERR_UNSUPPORTED = 3 };
 enum { TXS_F32 = 0, TXS_F16 = 1, TXS_BF16 = 2 };
-enum { TXS_SUM = 0, TXS_MEAN = 1, TXS_MAX = 2 };
+enum { TXS_SUM = 0, TXS_MEAN = 1, TXS_MAX = 2, TXS_MAX_REFTIE = 3 };
 
 /* Slots of the int32[TXS_STATS_LEN] device array the plan functions fill. */
 enum {
@@ -134,13 +134,20 @@ int txs_plan_seg_from_presum(const int32_t *preSum, int64_t num_total, int64_t n
  *     wins; a voxel with no non-NaN entry (or no rows) gets the lowest finite
  *     value of the dtype and arg = -1 (the reference's (-FLT_MAX, -1) init,
  *     scatter_kernel.cu:139-140).
+ *   op TXS_MAX_REFTIE: same values; among equal maxima the winner is the row
+ *     the reference kernel itself would report for the voxel's rows taken in
+ *     ascending order with block width clamp(up_2n(max_cnt), 32, 1024)
+ *     (scatter_kernel.cu:41-83,146-152,187: last row of a thread's residue
+ *     class, then smallest bit-reversed lane, then smallest bit-reversed warp);
+ *     -inf never wins, as in the reference.  max_cnt is the largest voxel
+ *     population (the reference launcher's argument); other ops ignore it.
  * out (and arg) need no initialisation: every element is written.
  * scratch may be NULL when num_special == 0. */
 int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *perm,
                         const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
                         const int32_t *heavy_ids, int64_t num_special, void *scratch,
                         void *out, int32_t *arg, int64_t num_total, int64_t channel,
-                        int64_t num_unq, void *stream);
+                        int64_t num_unq, int64_t max_cnt, void *stream);
 
 /* Backward as one gather pass over the sorted positions.  Replaces the ATen
  * ops of ScatterSumFunction.backward (scatter_op.py:47-50: g[unq_inv]),

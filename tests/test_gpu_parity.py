@@ -463,7 +463,7 @@ def test_c_abi_direct_call():
         ctypes.c_int(2), ctypes.c_int(0), vp(f.data_ptr()), vp(data.perm.data_ptr()), vp(data.seg.data_ptr()),
         vp(data.preSum.data_ptr()), vp(data.slot_of.data_ptr()),
         vp(data.heavy_ids.data_ptr() if data.num_special else 0), i64(data.num_special), vp(scratch.data_ptr()),
-        vp(out.data_ptr()), vp(arg.data_ptr()), i64(N), i64(C), i64(U), stream)
+        vp(out.data_ptr()), vp(arg.data_ptr()), i64(N), i64(C), i64(U), i64(data.max_cnt), stream)
     assert rc == 0
     torch.cuda.synchronize()
     wm, wa = orc.scatter_max_first(feats.numpy(), inv.numpy().astype(np.int32), U)
@@ -481,9 +481,80 @@ def test_c_abi_direct_call():
     # argument validation returns a status instead of launching
     rc = lib.txs_scatter_forward(
         ctypes.c_int(7), ctypes.c_int(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0), vp(0),
-        i64(N), i64(C), i64(U), stream)
+        i64(N), i64(C), i64(U), i64(1), stream)
     assert rc == 3
     rc = lib.txs_scatter_forward(
         ctypes.c_int(0), ctypes.c_int(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0), vp(0),
-        i64(N), i64(C), i64(U), stream)
+        i64(N), i64(C), i64(U), i64(1), stream)
     assert rc == 1
+
+
+# ------------------------------------------- the reference's own tie rule ----
+
+def _tie_heavy_groups(seed, sizes, C):
+    g = torch.Generator().manual_seed(seed)
+    cnts = torch.tensor(sizes, dtype=torch.long)
+    inv = torch.repeat_interleave(torch.arange(len(sizes)), cnts)
+    feats = torch.randint(0, 3, (int(cnts.sum()), C), generator=g).float()   # many equal maxima
+    return feats, inv, cnts
+
+
+@pytest.mark.parametrize("sizes", [
+    [5, 17, 31, 32, 33, 64, 1, 2, 100, 7] * 20,                 # block width 128: one row per thread
+    [700, 33, 1024, 5, 900, 64, 65, 1] * 6,                     # width 1024, everything within one pass
+    [2050, 1500, 40, 4996, 100, 1025, 3000, 64, 7, 1100] * 2,   # width 1024, several rows per thread
+])
+def test_reference_tie_rule_mode(sizes):
+    """max_tie_rule='reference' reports, among equal maxima, the row the reference kernel
+    keeps (lane-exact emulation in the oracle), for sorted input directly and for
+    shuffled input through the stable sort; the raw scatter_ext.max entry point, which
+    receives max_cnt like the reference's, does the same."""
+    T = tx()
+    import scatter_ext
+    C = 12
+    feats, inv, cnts = _tie_heavy_groups(len(sizes), sizes, C)
+    U, N = len(sizes), feats.shape[0]
+    inv32 = inv.numpy().astype(np.int32)
+    say(f"[case] reference tie rule N={N} U={U} max_cnt={max(sizes)}")
+    want_max, want_arg = orc.scatter_max_reforder(feats.numpy(), inv32, U)
+    first_max, first_arg = orc.scatter_max_first(feats.numpy(), inv32, U)
+    assert (want_arg != first_arg).any()   # the two rules really differ on this data
+
+    data = T.ScatterData(inv.to(DEV), cnts.to(DEV), max_tie_rule="reference")
+    mx, arg = T.scatter_max(feats.to(DEV), data)
+    assert np.array_equal(arg.cpu().numpy(), want_arg)
+    assert bits_equal(mx.cpu().numpy(), want_max)
+    # the default rule on the same data
+    d1 = T.ScatterData(inv.to(DEV), cnts.to(DEV))
+    assert np.array_equal(T.scatter_max(feats.to(DEV), d1)[1].cpu().numpy(), first_arg)
+    # all rows through the register path as well (no heavy voxels)
+    d2 = T.ScatterData(inv.to(DEV), cnts.to(DEV), heavy_threshold=1 << 20, max_tie_rule="reference")
+    assert np.array_equal(T.scatter_max(feats.to(DEV), d2)[1].cpu().numpy(), want_arg)
+
+    # the reference module's entry point on the sorted rows
+    out = torch.zeros((U, C), device=DEV)
+    a = torch.zeros((U, C), device=DEV, dtype=torch.int32)
+    scatter_ext.max(feats.to(DEV), data.preSum, out, a, data.max_cnt)
+    assert np.array_equal(a.cpu().numpy(), want_arg) and bits_equal(out.cpu().numpy(), want_max)
+
+    # shuffled rows: winner = reference rule on the stably sorted voxel, as original row ids
+    p = torch.randperm(N, generator=torch.Generator().manual_seed(5))
+    want_max_s, want_arg_s = orc.scatter_max_reforder(feats[p].numpy(), inv32[p.numpy()], U)
+    ds = T.ScatterData(inv[p].to(DEV), cnts.to(DEV), max_tie_rule="reference")
+    mx, arg = T.scatter_max(feats[p].to(DEV).requires_grad_(True), ds)
+    assert np.array_equal(arg.cpu().numpy(), want_arg_s)
+    assert bits_equal(mx.detach().cpu().numpy(), want_max_s)
+    # backward follows whichever arg was reported
+    gup = workloads.upstream_grad(U, C, 9)
+    x = feats[p].to(DEV).requires_grad_(True)
+    T.scatter_max(x, ds)[0].backward(gup.to(DEV))
+    assert bits_equal(x.grad.cpu().numpy(), orc.max_backward(gup.numpy(), want_arg_s, N))
+
+
+def test_reference_tie_rule_mode_matches_default_without_ties():
+    T = tx()
+    w = workloads.lidar_sweep(N=200_000, C=32, seed=12)
+    f = w.feats.to(DEV)
+    a = T.scatter_max(f, T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV)))
+    b = T.scatter_max(f, T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV), max_tie_rule="reference"))
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])

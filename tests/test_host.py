@@ -31,7 +31,7 @@ def test_header_symbols_are_exported():
 
 def test_host_only_entry_points():
     lib = _lib()
-    assert lib.txs_abi_version() == 2
+    assert lib.txs_abi_version() == 3
     lib.txs_status_string.restype = ctypes.c_char_p
     assert lib.txs_status_string(0) == b"ok"
     assert b"invalid" in lib.txs_status_string(1)
@@ -47,13 +47,13 @@ def test_argument_validation_needs_no_gpu():
     lib = _lib()
     vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     rc = lib.txs_scatter_forward(ci(9), ci(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0),
-                                 vp(0), i64(1), i64(1), i64(1), vp(0))
+                                 vp(0), i64(1), i64(1), i64(1), i64(1), vp(0))
     assert rc == 3
     rc = lib.txs_scatter_forward(ci(0), ci(5), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0),
-                                 vp(0), i64(1), i64(1), i64(1), vp(0))
+                                 vp(0), i64(1), i64(1), i64(1), i64(1), vp(0))
     assert rc == 3
     rc = lib.txs_scatter_forward(ci(0), ci(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0),
-                                 vp(0), i64(1 << 40), i64(1), i64(1), vp(0))
+                                 vp(0), i64(1 << 40), i64(1), i64(1), i64(1), vp(0))
     assert rc == 1
     rc = lib.txs_scatter_backward(ci(2), ci(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(5), i64(4), i64(2),
                                   vp(0))

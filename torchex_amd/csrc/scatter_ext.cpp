@@ -145,7 +145,7 @@ Tensor make_scratch(int64_t num_special, int64_t C, const Tensor &like) {
 
 void run_forward(int op, const Tensor &feats, const OptTensor &perm, const Tensor &seg,
                  const Tensor &preSum, const Tensor &slot_of, const Tensor &heavy_ids,
-                 Tensor &scratch, Tensor &out, OptTensor &arg) {
+                 Tensor &scratch, Tensor &out, OptTensor &arg, int64_t max_cnt) {
     const int64_t N = feats.size(0), C = feats.size(1), U = preSum.numel() - 1;
     const int64_t S = heavy_ids.numel();
     TORCH_CHECK(seg.numel() == N, "plan was built for ", seg.numel(), " rows, feats has ", N);
@@ -161,16 +161,17 @@ void run_forward(int op, const Tensor &feats, const OptTensor &perm, const Tenso
         rc = txs_scatter_forward(op, dt, feats.data_ptr(), opt_i32p(perm), i32p(seg), i32p(preSum),
                                  i32p(slot_of), i32p(heavy_ids), S,
                                  S ? scratch.data_ptr() : nullptr, out.data_ptr(),
-                                 arg.has_value() ? arg->data_ptr<int32_t>() : nullptr, N, C, U, st);
+                                 arg.has_value() ? arg->data_ptr<int32_t>() : nullptr, N, C, U, max_cnt,
+                                 st);
     }
     check_status(rc, "scatter_forward");
 }
 
-// forward(op, feats, perm|None, seg, preSum, slot_of, heavy_ids, scratch) -> (out, arg|None)
+// forward(op, feats, perm|None, seg, preSum, slot_of, heavy_ids, scratch, max_cnt) -> (out, arg|None)
 std::tuple<Tensor, OptTensor> forward(int64_t op, const Tensor &feats, const OptTensor &perm,
                                       const Tensor &seg, const Tensor &preSum,
                                       const Tensor &slot_of, const Tensor &heavy_ids,
-                                      Tensor scratch) {
+                                      Tensor scratch, int64_t max_cnt) {
     check_dev(feats, "feats");
     TORCH_CHECK(feats.dim() == 2, "feats must be [num_total, channel]");
     check_i32(seg, "seg");
@@ -185,8 +186,8 @@ std::tuple<Tensor, OptTensor> forward(int64_t op, const Tensor &feats, const Opt
     const int64_t C = feats.size(1), U = preSum.numel() - 1;
     Tensor out = at::empty({U, C}, feats.options());
     OptTensor arg;
-    if (op == TXS_MAX) arg = at::empty({U, C}, feats.options().dtype(at::kInt));
-    run_forward((int)op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, out, arg);
+    if (op == TXS_MAX || op == TXS_MAX_REFTIE) arg = at::empty({U, C}, feats.options().dtype(at::kInt));
+    run_forward((int)op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, out, arg, max_cnt);
     return {out, arg};
 }
 
@@ -202,7 +203,7 @@ Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const 
     TORCH_CHECK(grad_out.size(0) == U, "grad_out has ", grad_out.size(0), " rows, plan has ", U, " voxels");
     TORCH_CHECK(seg.numel() == N, "plan row count mismatch");
     TORCH_CHECK(!perm.has_value() || perm->numel() == N, "perm length mismatch");
-    if (op == TXS_MAX) {
+    if (op == TXS_MAX || op == TXS_MAX_REFTIE) {
         TORCH_CHECK(arg.has_value(), "scatter_max backward needs arg");
         check_i32(*arg, "arg");
         TORCH_CHECK(arg->dim() == 2 && arg->size(0) == U && arg->size(1) == C, "arg must be [num_unq, channel]");
@@ -223,7 +224,7 @@ Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const 
 
 // ---- the reference module's three functions (scatter.cpp:20-64) ------------
 
-void csr_reduce(int op, Tensor feats, Tensor preSum, Tensor out, OptTensor arg) {  // arg by value
+void csr_reduce(int op, Tensor feats, Tensor preSum, Tensor out, OptTensor arg, int64_t max_cnt) {
     check_dev(feats, "feats");
     check_i32(preSum, "preSum");
     check_dev(out, "out");
@@ -235,19 +236,22 @@ void csr_reduce(int op, Tensor feats, Tensor preSum, Tensor out, OptTensor arg) 
         plan_from_presum(preSum, feats.size(0), txs_default_heavy_threshold());
     Tensor scratch = make_scratch(heavy_ids.numel(), feats.size(1), feats);
     OptTensor perm;
-    run_forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, out, arg);
+    run_forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, out, arg, max_cnt);
 }
 
 // sum(feats, preSum, out, max_cnt): max_cnt only shaped the reference's thread
-// blocks (scatter_kernel.cu:179); it is accepted and not needed here.
-void sum_ref(Tensor feats, Tensor preSum, Tensor out, int64_t /*max_cnt*/) {
-    csr_reduce(TXS_SUM, feats, preSum, out, std::nullopt);
+// blocks (scatter_kernel.cu:179); it does not change a sum and is not needed here.
+void sum_ref(Tensor feats, Tensor preSum, Tensor out, int64_t max_cnt) {
+    csr_reduce(TXS_SUM, feats, preSum, out, std::nullopt, max_cnt);
 }
 
-void max_ref(Tensor feats, Tensor preSum, Tensor out, Tensor arg, int64_t /*max_cnt*/) {
+// max(feats, preSum, out, arg, max_cnt): the reference module's own entry point.
+// max_cnt selected the reference's block width (scatter_kernel.cu:187) and with
+// it the row reported among equal maxima; the same row is reported here.
+void max_ref(Tensor feats, Tensor preSum, Tensor out, Tensor arg, int64_t max_cnt) {
     check_i32(arg, "arg");
     TORCH_CHECK(arg.sizes() == out.sizes(), "arg must have the shape of out");
-    csr_reduce(TXS_MAX, feats, preSum, out, arg);
+    csr_reduce(TXS_MAX_REFTIE, feats, preSum, out, arg, max_cnt);
 }
 
 void get_presum_ref(Tensor unq_inv, Tensor preSum) {
@@ -268,11 +272,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("build_plan", &build_plan, "build_plan(unq_inv, num_unq, heavy_threshold, unq_cnts|None)");
     m.def("plan_from_presum", &plan_from_presum, "index preparation from CSR offsets");
     m.def("make_scratch", &make_scratch, "zeroed scratch table for the special voxels");
-    m.def("forward", &forward, "forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch)");
+    m.def("forward", &forward, "forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, max_cnt)");
     m.def("backward", &backward, "backward(op, grad_out, arg, perm, seg, preSum, num_total)");
     m.def("abi_version", &txs_abi_version);
     m.def("default_heavy_threshold", &txs_default_heavy_threshold);
     m.attr("SUM") = (int)TXS_SUM;
     m.attr("MEAN") = (int)TXS_MEAN;
     m.attr("MAX") = (int)TXS_MAX;
+    m.attr("MAX_REFTIE") = (int)TXS_MAX_REFTIE;
 }

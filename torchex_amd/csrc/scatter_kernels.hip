@@ -470,13 +470,40 @@ __global__ void seg_from_presum_kernel(const int *__restrict__ preSum, long n, i
 constexpr int kMargin = 64;           // staged entries past the tile's end
 constexpr int kNoSeg = 0x7fffffff;    // never a valid seg value
 
+// ---- the reference's winner among equal maxima (op TXS_MAX_REFTIE) ----------
+// scatter_kernel.cu:131-171 runs B = clamp(up_2n(max_cnt), 32, 1024) threads per
+// voxel; thread tid keeps the LAST maximal row of its residue class (rel % B ==
+// tid, '>=' at :148) and the shuffle trees (:41-83, strict '>') let the
+// candidate with the smallest bit-reversed lane index, then the smallest
+// bit-reversed warp index, survive.  A row at offset `rel` inside its voxel
+// therefore competes with the key below (smaller wins).
+constexpr int kIterBits = 21;
+constexpr unsigned kIterMask = (1u << kIterBits) - 1u;
+__device__ __forceinline__ unsigned ref_prio(unsigned tid, int wbits) {
+    const unsigned lane = __brev(tid & 31u) >> 27;
+    const unsigned warp = wbits > 0 ? (__brev(tid >> 5) >> (32 - wbits)) : 0u;
+    return (warp << 5) | lane;
+}
+__device__ __forceinline__ int ref_key(int rel, int blog2) {
+    const unsigned tid = (unsigned)rel & ((1u << blog2) - 1u);
+    const unsigned iter = ((unsigned)rel >> blog2) & kIterMask;
+    return (int)((ref_prio(tid, blog2 - 5) << kIterBits) | (kIterMask - iter));
+}
+__device__ __forceinline__ int ref_rel(int key, int blog2) {  // inverse of ref_key
+    const unsigned iter = kIterMask - ((unsigned)key & kIterMask);
+    return (int)((iter << blog2) | ref_prio((unsigned)key >> kIterBits, blog2 - 5));
+}
+
 template <class TR, int VEC, int OP>
 __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     const typename TR::raw *__restrict__ feats, const int *__restrict__ perm,
     const int *__restrict__ seg, const int *__restrict__ slot_of,
     typename TR::raw *__restrict__ out, int *__restrict__ arg,
-    unsigned long long *__restrict__ scratch, int N, int C, int U, int lpr_log2) {
+    unsigned long long *__restrict__ scratch, const int *__restrict__ preSum, int N, int C, int U,
+    int lpr_log2, int ref_log2) {
     using raw = typename TR::raw;
+    constexpr bool kMax = OP == TXS_MAX || OP == TXS_MAX_REFTIE;
+    constexpr bool kRef = OP == TXS_MAX_REFTIE;  // idx[] then holds ref_key, not a row
     extern __shared__ int lds[];
     const int G = kThreads >> lpr_log2;
     const int T = G * kChunk;
@@ -486,7 +513,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     // Partials of heavy voxels: two slots per lane group (a chunk can touch at
     // most two heavy runs, one at each end), combined across the workgroup
     // before anything goes to the global scratch table.
-    using SlotT = typename std::conditional<OP == TXS_MAX, unsigned long long, float>::type;
+    using SlotT = typename std::conditional<kMax, unsigned long long, float>::type;
     int *slot_id = perm_s + (n_seg_s - 1);
     SlotT *slot_val = reinterpret_cast<SlotT *>(lds + ((2 * n_seg_s - 1 + 2 * G + 1) & ~1));
     const int W = VEC << lpr_log2;        // elements per slot
@@ -549,13 +576,24 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     }
     const int lb_fast = min(lb, n_seg_s);  // end of the part whose ids are staged in LDS
 
+    // Start value of a running max: -inf, or in reference-tie mode the
+    // reference's own -FLT_MAX (scatter_kernel.cu:139), which -inf never beats.
+    const float acc0 = kRef ? TR::to_f(TR::lowest()) : (kMax ? -__builtin_inff() : 0.0f);
+    // offset of position l inside its voxel, for the reference's tie key; an
+    // ordinary run always starts inside the range, a heavy one may not
+    auto rel_of_run_start = [&](int sg, int l) -> int {
+        if (!kRef || sg >= 0) return 0;
+        const int u = sg & kIdMask;
+        return ((unsigned)u < (unsigned)U) ? (t0 - 1 + l) - preSum[u] : 0;
+    };
     float acc[VEC];
     int idx[VEC];
     int cur = seg_s[la];
     int run_l0 = la;
+    int rel0 = rel_of_run_start(cur, la);
 #pragma unroll
     for (int k = 0; k < VEC; ++k) {
-        acc[k] = (OP == TXS_MAX) ? -__builtin_inff() : 0.0f;
+        acc[k] = acc0;
         idx[k] = -1;
     }
 
@@ -563,7 +601,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     auto flush = [&](int run_end) {
         const int u = cur & kIdMask;
         if ((unsigned)u >= (unsigned)U) return;
-        if (OP == TXS_MAX) {
+        if (kMax && !kRef) {
             bool missing = false;
 #pragma unroll
             for (int k = 0; k < VEC; ++k) missing |= idx[k] < 0;
@@ -596,6 +634,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                 for (int k = 0; k < VEC; ++k) {
                     r.v[k] = idx[k] >= 0 ? TR::from_f(acc[k]) : TR::lowest();
                     ai.v[k] = idx[k];
+                    if (kRef && idx[k] >= 0) ai.v[k] = row_at(run_l0 + ref_rel(idx[k], ref_log2) - rel0);
                 }
                 st_stream<int, VEC>(arg + o, ai);
             }
@@ -607,7 +646,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
             SlotT *sv = slot_val + (size_t)sidx * W + lane_in * VEC;
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
-                if constexpr (OP == TXS_MAX) {
+                if constexpr (kMax) {
                     sv[k] = idx[k] >= 0 ? (((unsigned long long)ordered_bits(acc[k]) << 32) |
                                            (unsigned long long)(0xffffffffu - (unsigned)idx[k]))
                                         : 0ull;
@@ -628,19 +667,25 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
             flush(l);
             cur = sg;
             run_l0 = l;
+            rel0 = rel_of_run_start(sg, l);
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
-                acc[k] = (OP == TXS_MAX) ? -__builtin_inff() : 0.0f;
+                acc[k] = acc0;
                 idx[k] = -1;
             }
         }
+        const int tag = kRef ? ref_key(rel0 + (l - run_l0), ref_log2) : row;
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
             const float x = TR::to_f(v.v[k]);
-            if (OP == TXS_MAX) {
-                const bool take = valid && x > acc[k];  // strict: first row wins ties, NaN never wins
+            if (kMax) {
+                // strict '>': the first row wins ties, NaN never wins.  Reference-tie
+                // mode also takes an equal value whose key is smaller.
+                bool take = x > acc[k];
+                if (kRef) take |= (x == acc[k]) && ((unsigned)tag < (unsigned)idx[k]);
+                take &= valid;
                 acc[k] = take ? x : acc[k];
-                idx[k] = take ? row : idx[k];
+                idx[k] = take ? tag : idx[k];
             } else {
                 acc[k] += valid ? x : 0.0f;
             }
@@ -730,7 +775,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 const SlotT x = slot_val[(size_t)t * W + lane_in * VEC + k];
-                if constexpr (OP == TXS_MAX) tot[k] = x > tot[k] ? x : tot[k];
+                if constexpr (kMax) tot[k] = x > tot[k] ? x : tot[k];
                 else tot[k] += x;
             }
         }
@@ -739,7 +784,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
         const size_t o = (size_t)slot * C + col;
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
-            if constexpr (OP == TXS_MAX) {
+            if constexpr (kMax) {
                 if (tot[k] != 0ull) atomicMax(scratch + o + k, tot[k]);
             } else {
                 unsafeAtomicAdd(reinterpret_cast<float *>(scratch) + o + k, tot[k]);
@@ -755,17 +800,22 @@ __global__ void scatter_finalize_kernel(const typename TR::raw *__restrict__ fea
                                         const int *__restrict__ heavy_ids,
                                         unsigned long long *__restrict__ scratch,
                                         typename TR::raw *__restrict__ out,
-                                        int *__restrict__ arg, int n_special, int N, int C, int U) {
+                                        int *__restrict__ arg, int n_special, int N, int C, int U,
+                                        const int *__restrict__ perm, int ref_log2) {
     const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= (long)n_special * C) return;
     const int s = (int)(t / C), c = (int)(t - (long)s * C);
     const int u = heavy_ids[s];
     if ((unsigned)u >= (unsigned)U) return;
     const size_t o = (size_t)u * C + c;
-    if (OP == TXS_MAX) {
+    if (OP == TXS_MAX || OP == TXS_MAX_REFTIE) {
         const unsigned long long key = scratch[t];
         scratch[t] = 0ull;
-        const unsigned row = 0xffffffffu - (unsigned)(key & 0xffffffffull);
+        unsigned row = 0xffffffffu - (unsigned)(key & 0xffffffffull);
+        if (OP == TXS_MAX_REFTIE && key != 0ull) {  // the low word holds a tie key, not a row
+            const long pos = (long)preSum[u] + ref_rel((int)row, ref_log2);
+            row = (pos >= 0 && pos < N) ? (unsigned)(perm ? perm[pos] : (int)pos) : 0xffffffffu;
+        }
         if (key == 0ull || row >= (unsigned)N) {
             out[o] = TR::lowest();
             arg[o] = -1;
@@ -940,24 +990,29 @@ Geometry make_geometry(long N, long C, int elem, const void *p0, const void *p1,
 template <class TR, int VEC>
 hipError_t launch_fwd_op(int op, const Geometry &geo, hipStream_t st, const void *feats,
                          const int *perm, const int *seg, const int *preSum, const int *slot_of,
-                         void *out, int *arg, void *scratch, int N, int C, int U) {
+                         void *out, int *arg, void *scratch, int N, int C, int U, int ref_log2) {
     using raw = typename TR::raw;
     auto f = (const raw *)feats;
     auto o = (raw *)out;
     auto s = (unsigned long long *)scratch;
     dim3 blk(kThreads);
+    const unsigned lds4 = geo.lds_fwd_idx + 4 * geo.lds_slots, lds8 = geo.lds_fwd_idx + 8 * geo.lds_slots;
     switch (op) {
         case TXS_SUM:
-            scatter_fwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, geo.lds_fwd_idx + 4 * geo.lds_slots, st>>>(
-                f, perm, seg, slot_of, o, arg, s, N, C, U, geo.lpr_log2);
+            scatter_fwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, lds4, st>>>(
+                f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
             break;
         case TXS_MEAN:
-            scatter_fwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, geo.lds_fwd_idx + 4 * geo.lds_slots, st>>>(
-                f, perm, seg, slot_of, o, arg, s, N, C, U, geo.lpr_log2);
+            scatter_fwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, lds4, st>>>(
+                f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
+            break;
+        case TXS_MAX_REFTIE:
+            scatter_fwd_kernel<TR, VEC, TXS_MAX_REFTIE><<<geo.grid, blk, lds8, st>>>(
+                f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
             break;
         default:
-            scatter_fwd_kernel<TR, VEC, TXS_MAX><<<geo.grid, blk, geo.lds_fwd_idx + 8 * geo.lds_slots, st>>>(
-                f, perm, seg, slot_of, o, arg, s, N, C, U, geo.lpr_log2);
+            scatter_fwd_kernel<TR, VEC, TXS_MAX><<<geo.grid, blk, lds8, st>>>(
+                f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
             break;
     }
     return hipGetLastError();
@@ -966,12 +1021,12 @@ hipError_t launch_fwd_op(int op, const Geometry &geo, hipStream_t st, const void
 template <class TR>
 hipError_t launch_fwd(int op, const Geometry &geo, hipStream_t st, const void *feats,
                       const int *perm, const int *seg, const int *preSum, const int *slot_of,
-                      void *out, int *arg, void *scratch, int N, int C, int U) {
+                      void *out, int *arg, void *scratch, int N, int C, int U, int ref_log2) {
     constexpr int e = (int)sizeof(typename TR::raw);
 #define TXS_FWD(VB)                                                                              \
     if (geo.vec_bytes == VB)                                                                     \
         return launch_fwd_op<TR, (VB) / e>(op, geo, st, feats, perm, seg, preSum, slot_of, out,  \
-                                           arg, scratch, N, C, U);
+                                           arg, scratch, N, C, U, ref_log2);
     TXS_FWD(16)
     TXS_FWD(8)
     TXS_FWD(4)
@@ -985,7 +1040,7 @@ hipError_t launch_fwd(int op, const Geometry &geo, hipStream_t st, const void *f
 template <class TR>
 hipError_t launch_finalize(int op, hipStream_t st, const void *feats, const int *preSum,
                            const int *heavy_ids, void *scratch, void *out, int *arg,
-                           long n_special, int N, int C, int U) {
+                           long n_special, int N, int C, int U, const int *perm, int ref_log2) {
     using raw = typename TR::raw;
     const long total = n_special * C;
     if (total <= 0) return hipSuccess;
@@ -996,15 +1051,19 @@ hipError_t launch_finalize(int op, hipStream_t st, const void *feats, const int 
     switch (op) {
         case TXS_SUM:
             scatter_finalize_kernel<TR, TXS_SUM><<<grid, blk, 0, st>>>(f, preSum, heavy_ids, s, o, arg,
-                                                                      (int)n_special, N, C, U);
+                                                                      (int)n_special, N, C, U, perm, ref_log2);
             break;
         case TXS_MEAN:
-            scatter_finalize_kernel<TR, TXS_MEAN><<<grid, blk, 0, st>>>(f, preSum, heavy_ids, s, o,
-                                                                       arg, (int)n_special, N, C, U);
+            scatter_finalize_kernel<TR, TXS_MEAN><<<grid, blk, 0, st>>>(f, preSum, heavy_ids, s, o, arg,
+                                                                       (int)n_special, N, C, U, perm, ref_log2);
+            break;
+        case TXS_MAX_REFTIE:
+            scatter_finalize_kernel<TR, TXS_MAX_REFTIE><<<grid, blk, 0, st>>>(
+                f, preSum, heavy_ids, s, o, arg, (int)n_special, N, C, U, perm, ref_log2);
             break;
         default:
             scatter_finalize_kernel<TR, TXS_MAX><<<grid, blk, 0, st>>>(f, preSum, heavy_ids, s, o, arg,
-                                                                      (int)n_special, N, C, U);
+                                                                      (int)n_special, N, C, U, perm, ref_log2);
             break;
     }
     return hipGetLastError();
@@ -1072,7 +1131,7 @@ int radix_bits(int64_t U) {
 
 extern "C" {
 
-int txs_abi_version(void) { return 2; }
+int txs_abi_version(void) { return 3; }
 
 const char *txs_status_string(int status) {
     switch (status) {
@@ -1196,14 +1255,19 @@ int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *per
                         const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
                         const int32_t *heavy_ids, int64_t num_special, void *scratch, void *out,
                         int32_t *arg, int64_t num_total, int64_t channel, int64_t num_unq,
-                        void *stream) {
-    if (op != TXS_SUM && op != TXS_MEAN && op != TXS_MAX) return TXS_ERR_UNSUPPORTED;
+                        int64_t max_cnt, void *stream) {
+    if (op != TXS_SUM && op != TXS_MEAN && op != TXS_MAX && op != TXS_MAX_REFTIE)
+        return TXS_ERR_UNSUPPORTED;
     if (dtype != TXS_F32 && dtype != TXS_F16 && dtype != TXS_BF16) return TXS_ERR_UNSUPPORTED;
     if (!fits_i32(num_total) || !fits_i32(num_unq) || !fits_i32(channel) || num_special < 0 ||
         num_special > num_unq)
         return TXS_ERR_INVALID_ARG;
     if (num_unq == 0 || channel == 0) return TXS_OK;
-    if (!out || !preSum || (op == TXS_MAX && !arg)) return TXS_ERR_INVALID_ARG;
+    const bool is_max = op == TXS_MAX || op == TXS_MAX_REFTIE;
+    if (!out || !preSum || (is_max && !arg)) return TXS_ERR_INVALID_ARG;
+    // block width the reference would launch for this max_cnt (scatter_kernel.cu:187)
+    int ref_log2 = 5;
+    while (ref_log2 < 10 && (1LL << ref_log2) < max_cnt) ++ref_log2;
     if (num_total > 0 && (!feats || !seg || !slot_of)) return TXS_ERR_INVALID_ARG;
     if (num_special > 0 && (!scratch || !heavy_ids)) return TXS_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
@@ -1211,22 +1275,22 @@ int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *per
     const int elem = dtype == TXS_F32 ? 4 : 2;
     hipError_t e = hipSuccess;
     if (N > 0) {
-        Geometry geo = make_geometry(N, C, elem, feats, out, nullptr, op == TXS_MAX, arg);
+        Geometry geo = make_geometry(N, C, elem, feats, out, nullptr, is_max, arg);
         if (dtype == TXS_F32)
-            e = launch_fwd<F32>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U);
+            e = launch_fwd<F32>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U, ref_log2);
         else if (dtype == TXS_F16)
-            e = launch_fwd<F16>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U);
+            e = launch_fwd<F16>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U, ref_log2);
         else
-            e = launch_fwd<BF16>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U);
+            e = launch_fwd<BF16>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U, ref_log2);
         if (e != hipSuccess) return TXS_ERR_LAUNCH;
     }
     if (num_special > 0) {
         if (dtype == TXS_F32)
-            e = launch_finalize<F32>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U);
+            e = launch_finalize<F32>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U, perm, ref_log2);
         else if (dtype == TXS_F16)
-            e = launch_finalize<F16>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U);
+            e = launch_finalize<F16>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U, perm, ref_log2);
         else
-            e = launch_finalize<BF16>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U);
+            e = launch_finalize<BF16>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U, perm, ref_log2);
     }
     return status_of(e);
 }
@@ -1235,6 +1299,7 @@ int txs_scatter_backward(int op, int dtype, const void *grad_out, const int32_t 
                          const int32_t *perm, const int32_t *seg, const int32_t *preSum,
                          void *grad_in, int64_t num_total, int64_t channel, int64_t num_unq,
                          void *stream) {
+    if (op == TXS_MAX_REFTIE) op = TXS_MAX;  // the backward only reads arg
     if (op != TXS_SUM && op != TXS_MEAN && op != TXS_MAX) return TXS_ERR_UNSUPPORTED;
     if (dtype != TXS_F32 && dtype != TXS_F16 && dtype != TXS_BF16) return TXS_ERR_UNSUPPORTED;
     if (!fits_i32(num_total) || !fits_i32(num_unq) || !fits_i32(channel)) return TXS_ERR_INVALID_ARG;

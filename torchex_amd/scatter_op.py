@@ -35,7 +35,7 @@ class ScatterData:
     atomics), ``slot_of`` / ``heavy_ids`` (table of those voxels).
     """
 
-    def __init__(self, unq_inv, unq_cnts, heavy_threshold=None) -> None:
+    def __init__(self, unq_inv, unq_cnts, heavy_threshold=None, max_tie_rule="first") -> None:
         assert unq_inv.ndim in (
             1, 2), f"unq_inv in ScatterData should be 1 or 2-dims, but got {unq_inv.ndim}-dims"
         assert unq_cnts.ndim in (
@@ -45,6 +45,11 @@ class ScatterData:
             self.unq_cnts = unq_cnts.unsqueeze(-1)
         else:
             self.unq_cnts = unq_cnts
+        if max_tie_rule not in ("first", "reference"):
+            raise ValueError("max_tie_rule must be 'first' or 'reference'")
+        # which row scatter_max reports among equal maxima: the smallest row
+        # index, or the row the reference kernel's shuffle tree would keep
+        self.max_tie_rule = max_tie_rule
         if heavy_threshold is None:
             heavy_threshold = scatter_ext.default_heavy_threshold()
         self.heavy_threshold = int(heavy_threshold)
@@ -84,7 +89,7 @@ def _check_feats(feats, data):
 def _forward(op, feats, data):
     _check_feats(feats, data)
     return scatter_ext.forward(op, feats, data.perm, data.seg, data.preSum, data.slot_of,
-                               data.heavy_ids, data.scratch(feats.shape[1]))
+                               data.heavy_ids, data.scratch(feats.shape[1]), data.max_cnt)
 
 
 def _backward(op, g, arg, data):
@@ -134,10 +139,13 @@ class ScatterMaxFunction(Function):
     def forward(ctx, feats: torch.Tensor, data: ScatterData):
         """scatter_max forward (``scatter_op.py:84-103``).
         Returns ``(out [num_unq, channel], arg [num_unq, channel] int32)`` where
-        ``arg`` is the row index into ``feats`` of the winning element (the
-        smallest such row when several rows tie).
+        ``arg`` is the row index into ``feats`` of the winning element.  When
+        several rows tie, the smallest row wins (``data.max_tie_rule ==
+        "first"``, the default) or the row the reference kernel would report
+        for the voxel's rows in ascending order (``"reference"``).
         """
-        out, arg = _forward(_MAX, feats, data)
+        op = scatter_ext.MAX_REFTIE if data.max_tie_rule == "reference" else _MAX
+        out, arg = _forward(op, feats, data)
         ctx.save_for_backward(arg)
         ctx.mark_non_differentiable(arg)
         # no zero tensor is made for the gradient slot of the integer output
