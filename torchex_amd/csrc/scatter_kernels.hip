@@ -750,45 +750,71 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     };  // reduce_chunk
     reduce_chunk();
 
-    // Workgroup-level merge of the parked partials: the used slots that carry
+    // Workgroup-level merge of the parked partials.  The used slots that carry
     // the same voxel id form one range (a heavy run is contiguous in sorted
-    // order, so only unused slots can sit between them); the first slot's lane
-    // group folds the range in slot order and issues one atomic per element.
-    // Tiles without a heavy voxel skip this phase and its barrier.
+    // order, so only unused slots can sit between them).  All 256 threads take
+    // part: (A) mark the first slot of every range, (B) fold every other slot
+    // into its range's first slot with LDS atomics, (C) send each range total to
+    // the global table with one atomic per element.  Tiles without a heavy voxel
+    // skip all of this and its barriers.
     if (!tile_has_heavy) return;
+#if TXS_DIAG == 5
+    return;
+#endif
+    __shared__ unsigned long long start_mask[(2 * kThreads) / 64];
+    const int S = 2 * G;                       // slots in this workgroup
+    const int w_log2 = lpr_log2 + (VEC == 8 ? 3 : VEC == 4 ? 2 : VEC == 2 ? 1 : 0);  // log2(W)
     __syncthreads();
-    if (col >= C) return;
-    for (int h = 0; h < 2; ++h) {
-        const int s0 = 2 * gi + h;
-        const int id = slot_id[s0];
-        if (id < 0) continue;
-        int prev = s0 - 1;
-        while (prev >= 0 && slot_id[prev] < 0) --prev;
-        if (prev >= 0 && slot_id[prev] == id) continue;  // not the first slot of its range
-        SlotT tot[VEC];
-#pragma unroll
-        for (int k = 0; k < VEC; ++k) tot[k] = slot_val[(size_t)s0 * W + lane_in * VEC + k];
-        for (int t = s0 + 1; t < 2 * G; ++t) {
-            const int tid = slot_id[t];
-            if (tid < 0) continue;
-            if (tid != id) break;
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) {
-                const SlotT x = slot_val[(size_t)t * W + lane_in * VEC + k];
-                if constexpr (kMax) tot[k] = x > tot[k] ? x : tot[k];
-                else tot[k] += x;
+    for (int base = 0; base < S; base += kThreads) {
+        const int sl = base + (int)threadIdx.x;
+        bool first = false;
+        if (sl < S) {
+            const int id = slot_id[sl];
+            if (id >= 0) {
+                int prev = sl - 1;
+                while (prev >= 0 && slot_id[prev] < 0) --prev;
+                first = prev < 0 || slot_id[prev] != id;
             }
         }
-        const int slot = slot_of[id];
+        const unsigned long long m = __ballot(first);
+        if ((threadIdx.x & 63) == 0) start_mask[(base + (int)threadIdx.x) >> 6] = m;
+    }
+    __syncthreads();
+    // first slot of the range that slot sl belongs to: nearest marked slot at or below sl
+    auto range_start = [&](int sl) -> int {
+        int wd = sl >> 6;
+        unsigned long long m = start_mask[wd] & (~0ull >> (63 - (sl & 63)));
+        while (m == 0ull && wd > 0) m = start_mask[--wd];
+        return m ? (wd << 6) + 63 - __builtin_clzll(m) : sl;
+    };
+    for (int i = threadIdx.x; i < (S << w_log2); i += kThreads) {
+        const int sl = i >> w_log2, e = i & (W - 1);
+        if (slot_id[sl] < 0) continue;
+        const int head = range_start(sl);
+        if (head == sl) continue;
+        const SlotT x = slot_val[i];
+        SlotT *dst = slot_val + ((size_t)head << w_log2) + e;
+        if constexpr (kMax) {
+            if (x != 0ull) atomicMax(dst, x);
+        } else {
+            __hip_atomic_fetch_add(dst, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < (S << w_log2); i += kThreads) {
+        const int sl = i >> w_log2, e = i & (W - 1);
+        if (!((start_mask[sl >> 6] >> (sl & 63)) & 1ull)) continue;
+        const int c = (((int)blockIdx.y << lpr_log2) * VEC) + e;
+        if (c >= C) continue;
+        const int id = slot_id[sl];
+        const int slot = ((unsigned)id < (unsigned)U) ? slot_of[id] : -1;
         if (slot < 0) continue;
-        const size_t o = (size_t)slot * C + col;
-#pragma unroll
-        for (int k = 0; k < VEC; ++k) {
-            if constexpr (kMax) {
-                if (tot[k] != 0ull) atomicMax(scratch + o + k, tot[k]);
-            } else {
-                unsafeAtomicAdd(reinterpret_cast<float *>(scratch) + o + k, tot[k]);
-            }
+        const SlotT tot = slot_val[i];
+        const size_t o = (size_t)slot * C + c;
+        if constexpr (kMax) {
+            if (tot != 0ull) atomicMax(scratch + o, tot);
+        } else {
+            unsafeAtomicAdd(reinterpret_cast<float *>(scratch) + o, tot);
         }
     }
 }
