@@ -319,22 +319,40 @@ __device__ __forceinline__ int wave_max_i32(int x) {
 }
 
 // Special-voxel table, max_cnt, and the check of the caller's counts against
-// the histogram.  One atomic per wavefront for the statistics.
-__global__ void plan_special_kernel(const int *__restrict__ preSum, int U, int heavy_threshold,
-                                    const long long *__restrict__ unq_cnts,
-                                    int *__restrict__ slot_of, int *__restrict__ heavy_ids,
-                                    int *__restrict__ stats) {
+// the histogram.  Launched with 1024-thread workgroups: the statistics are
+// reduced across the workgroup first, because device-scope atomics on one
+// address complete one after the other (~10 ns each) and one per wavefront
+// would dominate the kernel.
+constexpr int kSpecialThreads = 1024;
+__global__ __launch_bounds__(kSpecialThreads) void plan_special_kernel(
+    const int *__restrict__ preSum, int U, int heavy_threshold,
+    const long long *__restrict__ unq_cnts, int *__restrict__ slot_of,
+    int *__restrict__ heavy_ids, int *__restrict__ stats) {
+    __shared__ int s_max[kSpecialThreads / 64], s_empty[kSpecialThreads / 64], s_bad[kSpecialThreads / 64];
     const int u = blockIdx.x * blockDim.x + threadIdx.x;
     const bool in = u < U;
     const int c = in ? preSum[u + 1] - preSum[u] : 0;
     const int wmax = wave_max_i32(c);
     const int n_empty = __popcll(__ballot(in && c == 0));
     const bool mismatch = in && unq_cnts && unq_cnts[u] != (long long)c;
-    const bool any_mismatch = __ballot(mismatch) != 0ull;
+    const int any_mismatch = __ballot(mismatch) != 0ull;
+    const int w = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) {
-        if (wmax > 0) atomicMax(&stats[TXS_STAT_MAX_CNT], wmax);
-        if (n_empty) atomicAdd(&stats[TXS_STAT_NUM_EMPTY], n_empty);
-        if (any_mismatch) stats[TXS_STAT_COUNT_MISMATCH] = 1;
+        s_max[w] = wmax;
+        s_empty[w] = n_empty;
+        s_bad[w] = any_mismatch;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int m = 0, e = 0, b = 0;
+        for (int k = 0; k < kSpecialThreads / 64; ++k) {
+            m = max(m, s_max[k]);
+            e += s_empty[k];
+            b |= s_bad[k];
+        }
+        if (m > 0) atomicMax(&stats[TXS_STAT_MAX_CNT], m);
+        if (e) atomicAdd(&stats[TXS_STAT_NUM_EMPTY], e);
+        if (b) stats[TXS_STAT_COUNT_MISMATCH] = 1;
     }
     if (!in) return;
     int slot = -1;
@@ -1252,7 +1270,8 @@ int txs_plan_special(const int32_t *preSum, int64_t num_unq, int32_t heavy_thres
     if (!fits_i32(num_unq) || !preSum || !stats || heavy_threshold < kChunk) return TXS_ERR_INVALID_ARG;
     if (num_unq == 0) return TXS_OK;
     if (!slot_of || !heavy_ids) return TXS_ERR_INVALID_ARG;
-    plan_special_kernel<<<dim3(blocks_for(num_unq)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+    plan_special_kernel<<<dim3(blocks_for(num_unq, kSpecialThreads)), dim3(kSpecialThreads), 0,
+                          (hipStream_t)stream>>>(
         preSum, (int)num_unq, heavy_threshold, (const long long *)unq_cnts, slot_of, heavy_ids, stats);
     return status_of(hipGetLastError());
 }
