@@ -56,6 +56,7 @@ enum {
     TXS_STAT_NUM_SPECIAL = 3,  /* number of special voxels (heavy or empty) */
     TXS_STAT_NUM_EMPTY = 4,    /* number of voxels with zero rows */
     TXS_STAT_COUNT_MISMATCH = 5, /* 1 if the caller's unq_cnts is not the histogram of unq_inv */
+    TXS_STAT_NUM_UNQ = 6,      /* number of distinct keys found by txs_unique_runs */
     TXS_STATS_LEN = 8
 };
 
@@ -109,10 +110,14 @@ int txs_plan_presum(const int32_t *sorted_keys, int64_t num_total, int64_t num_u
  * stats[NUM_SPECIAL], stats[NUM_EMPTY]; when unq_cnts (int64 [num_unq], as
  * torch.unique returns it) is given, stats[COUNT_MISMATCH] is set if it is not
  * the histogram of unq_inv (the consistency check of scatter_op.py:19).
- * heavy_ids must hold num_unq entries (the first NUM_SPECIAL are used). */
+ * heavy_ids must hold num_unq entries (the first NUM_SPECIAL are used).
+ * num_unq_dev (may be NULL): device int holding the true voxel count when the
+ * host only knows the upper bound passed as num_unq (after txs_unique_runs).
+ * cnts_out (may be NULL): int64 [num_unq] voxel populations, the unq_cnts of
+ * torch.unique. */
 int txs_plan_special(const int32_t *preSum, int64_t num_unq, int32_t heavy_threshold,
                      const int64_t *unq_cnts, int32_t *slot_of, int32_t *heavy_ids, int32_t *stats,
-                     void *stream);
+                     const int32_t *num_unq_dev, int64_t *cnts_out, void *stream);
 
 /* In place: sorted keys -> seg (sets bit 31 on positions of special voxels). */
 int txs_plan_seg_flag(int32_t *keys_to_seg, int64_t num_total, int64_t num_unq,
@@ -123,6 +128,41 @@ int txs_plan_seg_flag(int32_t *keys_to_seg, int64_t num_total, int64_t num_unq,
  * scatter_ext.max argument lists, scatter.cpp:20-53). */
 int txs_plan_seg_from_presum(const int32_t *preSum, int64_t num_total, int64_t num_unq,
                              const int32_t *slot_of, int32_t *seg, void *stream);
+
+/* ---- callers on either side of the path ------------------------------------ */
+
+/* Dynamic voxelization front-end: per point, coors = floor((p - range_lo) /
+ * voxel_size) with the arithmetic of torch.div(..., rounding_mode='floor') on
+ * fp32 (the reference's voxelize_single, test/test_incremental_mask.py:20-26)
+ * and key = (x * dims[1] + y) * dims[2] + z (operator_py/incremental_points.py:
+ * 18-19, operator_py/grid_hash.py:14).  points: [num_total, point_stride] fp32,
+ * xyz first.  range_lo / voxel_size / dims are HOST arrays of 3.  coors (may be
+ * NULL): int32 [num_total, 3].  A point outside the grid sets
+ * stats[OUT_OF_RANGE] and gets key 0. */
+int txs_voxel_keys(const float *points, int64_t num_total, int64_t point_stride,
+                   const float *range_lo, const float *voxel_size, const int32_t *dims,
+                   int32_t *coors, int32_t *keys, int32_t *stats, void *stream);
+
+/* What torch.unique(keys, return_inverse=True, return_counts=True) computes,
+ * fused with the plan: from keys sorted by txs_plan_sort (called with the key
+ * bound in place of num_unq) it writes unq_keys [<= num_total] (ascending),
+ * unq_inv [num_total] (int32), preSum, seg (dense voxel id per sorted
+ * position) and stats[NUM_UNQ]; follow with txs_plan_special (num_unq_dev =
+ * &stats[NUM_UNQ], cnts_out for the counts) and txs_plan_seg_flag.  One sort
+ * serves both the unique and the scatter plan.  unique_ws: int32 workspace of
+ * txs_unique_workspace_len(num_total) entries. */
+int txs_unique_runs(const int32_t *sorted_keys, const int32_t *perm, int64_t num_total,
+                    int32_t *unique_ws, int32_t *seg, int32_t *unq_inv, int32_t *unq_keys,
+                    int32_t *preSum, int32_t *stats, void *stream);
+int64_t txs_unique_workspace_len(int64_t num_total);
+
+/* Rank of every element inside its group, from the plan of its group ids:
+ * out[row] = sorted position - preSum[group].  Replaces ingroup_inds_launcher
+ * (torchex/src/ingroup_inds/ingroup_inds.cpp:14-19, kernel
+ * ingroup_inds_kernel.cu:17-30); ranks ascend with the element index inside a
+ * group (the reference's atomic counter gives them in arbitrary order). */
+int txs_ingroup_inds(const int32_t *seg, const int32_t *perm, const int32_t *preSum,
+                     int64_t num_total, int64_t num_unq, int64_t *out, void *stream);
 
 /* ---- the hot path --------------------------------------------------------- */
 

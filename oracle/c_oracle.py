@@ -191,3 +191,23 @@ def scatter_max_reforder(feats, unq_inv, num_unq):
     out, arg = scatter_max_ref(fs, pre, int(cnt.max()) if cnt.size else 1)
     arg_rows = np.where(arg >= 0, perm[np.clip(arg, 0, None)] if perm.size else arg, -1).astype(np.int32)
     return out, arg_rows
+
+
+def ingroup_inds(group_ids):
+    g = _i64(group_ids)
+    out = np.empty_like(g)
+    if g.size:
+        lib().orc_ingroup_inds(_p(g), _ll(g.shape[0]), _ll(int(g.max())), _p(out))
+    return out
+
+
+def voxelize(points, voxel_size, range_lo, dims):
+    pts = _f32(points)
+    lo = _f32(range_lo)
+    vs = _f32(voxel_size)
+    dm = _i32(dims)
+    n = pts.shape[0]
+    coors = np.empty((n, 3), dtype=np.int32)
+    keys = np.empty(n, dtype=np.int32)
+    lib().orc_voxelize(_p(pts), _ll(n), _ll(pts.shape[1]), _p(lo), _p(vs), _p(dm), _p(coors), _p(keys))
+    return coors, keys

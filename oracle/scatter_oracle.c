@@ -339,3 +339,50 @@ void orc_max_backward(const float *g, const int32_t *arg, int64_t n, int64_t C, 
             if (r >= 0 && r < n) gin[(int64_t)r * C + c] = g[u * C + c];
         }
 }
+
+/* ---- callers on either side of the path -------------------------------- */
+
+/* ingroup_inds_kernel (torchex/src/ingroup_inds/ingroup_inds_kernel.cu:17-30):
+ * out[i] = atomicAdd(&counter[group[i]], 1).  The device hands the ranks of a
+ * group out in whatever order its threads arrive; here the threads run in
+ * index order, which is one of the possible outcomes and the one the HIP path
+ * always produces.  counter must hold max_group_id + 1 zeroed ints
+ * (ingroup_inds_kernel.cu:40-42). */
+void orc_ingroup_inds(const int64_t *group, int64_t n, int64_t max_group_id, int64_t *out) {
+    int32_t *counter = (int32_t *)calloc((size_t)(max_group_id + 1), sizeof(int32_t));
+    for (int64_t i = 0; i < n; ++i) out[i] = counter[group[i]]++;
+    free(counter);
+}
+
+/* c10::div_floor_floating<float> (what torch.div(a, b, rounding_mode='floor')
+ * applies per element): Python's floor division. */
+static float orc_div_floor(float a, float b) {
+    if (b == 0.0f) return a / b;
+    volatile float mod = fmodf(a, b);
+    volatile float div = (a - mod) / b;
+    if ((mod != 0.0f) && ((b < 0.0f) != (mod < 0.0f))) div = div - 1.0f;
+    float fl;
+    if (div != 0.0f) {
+        fl = floorf(div);
+        if (div - fl > 0.5f) fl += 1.0f;
+    } else {
+        fl = copysignf(0.0f, a / b);
+    }
+    return fl;
+}
+
+/* voxelize_single (test/test_incremental_mask.py:20-26):
+ * torch.div(points[:, :3] - pc_range[:3], voxel_size, rounding_mode='floor').int()
+ * and the x-major linear key of operator_py/incremental_points.py:18-19 */
+void orc_voxelize(const float *points, int64_t n, int64_t stride, const float *lo, const float *vs,
+                  const int32_t *dims, int32_t *coors, int32_t *keys) {
+    for (int64_t i = 0; i < n; ++i) {
+        int32_t c[3];
+        for (int a = 0; a < 3; ++a) {
+            volatile float d = points[i * stride + a] - lo[a];
+            c[a] = (int32_t)orc_div_floor(d, vs[a]);
+            coors[i * 3 + a] = c[a];
+        }
+        keys[i] = (c[0] * dims[1] + c[1]) * dims[2] + c[2];
+    }
+}

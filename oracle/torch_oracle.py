@@ -75,3 +75,17 @@ def step_mean_max(feats, unq_inv, unq_cnts, g_mean, g_max):
     mx, arg = scatter_max(feats, unq_inv, U)
     gi_max = max_backward(g_max, arg, feats.shape[0])
     return mean, gi_mean, mx, arg, gi_max
+
+
+def voxelize(points, voxel_size, pc_range):
+    """The reference's ``voxelize_single`` verbatim in spirit
+    (``test/test_incremental_mask.py:20-26``), on CPU tensors."""
+    vs = torch.tensor(voxel_size, dtype=torch.float32)
+    rng = torch.tensor(pc_range, dtype=torch.float32)
+    return torch.div(points[:, :3] - rng[None, :3], vs[None, :], rounding_mode='floor').int()
+
+
+def flatten_coors(coors, sizes):
+    """``operator_py/grid_hash.py:7-15`` / ``operator_py/incremental_points.py:18-19``."""
+    x, y, z = coors[:, 0].long(), coors[:, 1].long(), coors[:, 2].long()
+    return x * (sizes[1] * sizes[2]) + y * sizes[2] + z

@@ -342,3 +342,39 @@ def test_backward_against_torch_ops_and_autograd():
         .backward(g.double())
     # no ties in N(0,1) data: amax's gradient goes to the single winner
     assert np.array_equal(x.grad.float().numpy(), orc.max_backward(g.numpy(), a, w.N))
+
+
+# ------------------------------------------- callers on either side of the path --
+
+def test_ingroup_inds_oracle():
+    rng = np.random.default_rng(21)
+    g = rng.integers(0, 37, size=4000).astype(np.int64)
+    out = orc.ingroup_inds(g)
+    # what the reference guarantees: inside each group the ranks are 0..cnt-1, each once
+    for gid in range(37):
+        r = np.sort(out[g == gid])
+        assert np.array_equal(r, np.arange(r.shape[0]))
+    # in index order: rank = number of earlier elements of the same group (brute force)
+    brute = np.array([int((g[:i] == g[i]).sum()) for i in range(300)])
+    assert np.array_equal(out[:300], brute)
+
+
+def test_voxelize_oracle_against_torch_floor_division():
+    g = torch.Generator().manual_seed(31)
+    pts = torch.rand((20000, 4), generator=g) * 160.0 - 80.0
+    # points exactly on cell edges and just beside them, negative and positive
+    edges = torch.arange(-80.0, 80.0, 0.25)[:640]
+    pts[:640, 0] = edges
+    pts[640:1280, 1] = torch.nextafter(edges, torch.tensor(-1e9))
+    pts[1280:1920, 2] = torch.nextafter(edges, torch.tensor(1e9)) * 0.05
+    voxel_size, pc_range = [0.25, 0.25, 0.4], [-80, -80, -2, 80, 80, 4]
+    want = tor.voxelize(pts, voxel_size, pc_range).numpy()
+    coors, keys = orc.voxelize(pts.numpy(), voxel_size, pc_range[:3], [640, 640, 15])
+    assert np.array_equal(coors, want)
+    inr = ((want >= 0) & (want < np.array([640, 640, 15]))).all(1)
+    wk = tor.flatten_coors(torch.from_numpy(want), (640, 640, 15)).numpy()
+    assert np.array_equal(keys[inr], wk[inr].astype(np.int32))
+    # Python's floor division is not floor(a / b) in general; the textbook cases agree
+    for a, b in [(7.0, 2.0), (-7.0, 2.0), (7.0, -2.0), (0.3, 0.1), (-0.3, 0.1), (1.0, 0.1)]:
+        c, _ = orc.voxelize(np.array([[a, 0, 0]], np.float32), [b, 1, 1], [0, 0, 0], [1 << 20, 1, 1])
+        assert c[0, 0] == int(np.float32(a) // np.float32(b)), (a, b)

@@ -6,7 +6,8 @@ TorchTimer`` -- the names the reference exports for this path
 kernel library and the ``scatter_ext`` extension module and raises if either is
 missing.
 """
-from .scatter_op import ScatterData, getPreSum, scatter_max, scatter_mean, scatter_sum
+from .scatter_op import (ScatterData, getPreSum, ingroup_inds, scatter_max, scatter_mean, scatter_sum,
+                         voxelize)
 from .timer import TorchTimer
 
-__all__ = ['TorchTimer', 'scatter_sum', 'scatter_mean', 'scatter_max', 'ScatterData']
+__all__ = ['TorchTimer', 'scatter_sum', 'scatter_mean', 'scatter_max', 'ScatterData', 'ingroup_inds']

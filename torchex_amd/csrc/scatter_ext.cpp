@@ -103,7 +103,7 @@ std::tuple<Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>> buil
                      "plan_sort");
     check_status(txs_plan_presum(i32p(seg), U > 0 ? N : 0, U, i32w(preSum), st), "plan_presum");
     check_status(txs_plan_special(i32p(preSum), U, (int32_t)heavy_threshold, cnts, i32w(slot_of),
-                                  i32w(heavy_all), i32w(stats), st),
+                                  i32w(heavy_all), i32w(stats), nullptr, nullptr, st),
                  "plan_special");
     check_status(txs_plan_seg_flag(i32w(seg), U > 0 ? N : 0, U, i32p(slot_of), st), "plan_seg_flag");
     std::vector<int64_t> hs = read_stats(stats);
@@ -128,7 +128,7 @@ std::tuple<Tensor, Tensor, Tensor, std::vector<int64_t>> plan_from_presum(
     Tensor slot_of = empty_i32(U, preSum);
     Tensor heavy_all = empty_i32(U, preSum);
     check_status(txs_plan_special(i32p(preSum), U, (int32_t)heavy_threshold, nullptr, i32w(slot_of),
-                                  i32w(heavy_all), i32w(stats), st),
+                                  i32w(heavy_all), i32w(stats), nullptr, nullptr, st),
                  "plan_special");
     Tensor seg = empty_i32(N, preSum);
     if (U > 0)
@@ -137,6 +137,89 @@ std::tuple<Tensor, Tensor, Tensor, std::vector<int64_t>> plan_from_presum(
     std::vector<int64_t> hs = read_stats(stats);
     Tensor heavy_ids = heavy_all.narrow(0, 0, hs[TXS_STAT_NUM_SPECIAL]).contiguous();
     return {seg, slot_of, heavy_ids, hs};
+}
+
+// Dynamic voxelization front-end: coors and linear keys of every point; no host
+// synchronisation (range violations are flagged in the returned stats tensor).
+// returns (coors [N,3] int32, keys [N] int32, stats [TXS_STATS_LEN] int32)
+std::tuple<Tensor, Tensor, Tensor> voxel_keys(const Tensor &points, std::vector<double> range_lo,
+                                              std::vector<double> voxel_size,
+                                              std::vector<int64_t> dims) {
+    check_dev(points, "points");
+    TORCH_CHECK(points.dim() == 2 && points.size(1) >= 3, "points must be [N, >=3]");
+    TORCH_CHECK(points.scalar_type() == at::kFloat, "points must be float32");
+    TORCH_CHECK(range_lo.size() == 3 && voxel_size.size() == 3 && dims.size() == 3,
+                "range_lo, voxel_size and dims need 3 entries");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(points.device());
+    const int64_t N = points.size(0);
+    const float lo[3] = {(float)range_lo[0], (float)range_lo[1], (float)range_lo[2]};
+    const float vs[3] = {(float)voxel_size[0], (float)voxel_size[1], (float)voxel_size[2]};
+    const int32_t dm[3] = {(int32_t)dims[0], (int32_t)dims[1], (int32_t)dims[2]};
+    Tensor coors = at::empty({N, 3}, points.options().dtype(at::kInt));
+    Tensor keys = at::empty({N}, points.options().dtype(at::kInt));
+    Tensor stats = at::zeros({TXS_STATS_LEN}, points.options().dtype(at::kInt));
+    check_status(txs_voxel_keys(N ? points.data_ptr<float>() : nullptr, N, points.size(1), lo, vs, dm,
+                                i32w(coors), i32w(keys), i32w(stats), cur_stream(points)),
+                 "voxel_keys");
+    return {coors, keys, stats};
+}
+
+// torch.unique(keys, return_inverse=True, return_counts=True) fused with the
+// scatter plan: one sort, one host synchronisation.
+// returns (unq_keys, unq_inv, unq_cnts, preSum, perm | None, seg, slot_of, heavy_ids, stats)
+std::tuple<Tensor, Tensor, Tensor, Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>>
+unique_plan(const Tensor &keys, int64_t key_bound, int64_t heavy_threshold, const OptTensor &stats_in) {
+    check_i32(keys, "keys");
+    TORCH_CHECK(keys.dim() == 1, "keys must be 1-D");
+    TORCH_CHECK(key_bound > 0, "key_bound must be positive");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(keys.device());
+    const int64_t N = keys.numel();
+    void *st = cur_stream(keys);
+    Tensor stats = stats_in.has_value() ? *stats_in : at::zeros({TXS_STATS_LEN}, keys.options());
+    check_i32(stats, "stats");
+    TORCH_CHECK(stats.numel() == TXS_STATS_LEN, "stats must have TXS_STATS_LEN entries");
+    Tensor seg = empty_i32(N, keys), perm = empty_i32(N, keys), inv = empty_i32(N, keys);
+    Tensor unq = empty_i32(N, keys), preSum = empty_i32(N + 1, keys);
+    Tensor slot_of = empty_i32(N, keys), heavy_all = empty_i32(N, keys);
+    Tensor cnts = at::empty({N}, keys.options().dtype(at::kLong));
+    Tensor ws = empty_i32(txs_sort_workspace_len(N, key_bound), keys);
+    Tensor uws = empty_i32(txs_unique_workspace_len(N), keys);
+    check_status(txs_plan_check(i32p(keys), N, key_bound, i32w(stats), st), "plan_check");
+    Tensor sorted_keys = empty_i32(N, keys);  // unique_runs reads neighbours: not the same array as seg
+    check_status(txs_plan_sort(i32p(keys), N, key_bound, i32p(stats), i32w(perm), i32w(sorted_keys),
+                               i32w(ws), st),
+                 "plan_sort");
+    check_status(txs_unique_runs(i32p(sorted_keys), i32p(perm), N, i32w(uws), i32w(seg), i32w(inv),
+                                 i32w(unq), i32w(preSum), i32w(stats), st),
+                 "unique_runs");
+    const int32_t *u_dev = stats.data_ptr<int32_t>() + TXS_STAT_NUM_UNQ;
+    check_status(txs_plan_special(i32p(preSum), N, (int32_t)heavy_threshold, nullptr, i32w(slot_of),
+                                  i32w(heavy_all), i32w(stats), u_dev,
+                                  N ? cnts.data_ptr<int64_t>() : nullptr, st),
+                 "plan_special");
+    check_status(txs_plan_seg_flag(i32w(seg), N, N, i32p(slot_of), st), "plan_seg_flag");
+    std::vector<int64_t> hs = read_stats(stats);
+    TORCH_CHECK(hs[TXS_STAT_OUT_OF_RANGE] == 0, "keys (or points) outside the grid: keys must be in [0, ",
+                key_bound, ")");
+    const int64_t U = hs[TXS_STAT_NUM_UNQ];
+    OptTensor perm_out;
+    if (hs[TXS_STAT_UNSORTED]) perm_out = perm;
+    return {unq.narrow(0, 0, U), inv, cnts.narrow(0, 0, U), preSum.narrow(0, 0, U + 1), perm_out, seg,
+            slot_of.narrow(0, 0, U), heavy_all.narrow(0, 0, hs[TXS_STAT_NUM_SPECIAL]).contiguous(), hs};
+}
+
+// ingroup_inds(seg, perm | None, preSum, num_unq) -> int64 [N]
+Tensor ingroup_inds(const Tensor &seg, const OptTensor &perm, const Tensor &preSum, int64_t num_unq) {
+    check_i32(seg, "seg");
+    check_i32(preSum, "preSum");
+    if (perm.has_value()) check_i32(*perm, "perm");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(seg.device());
+    const int64_t N = seg.numel();
+    Tensor out = at::empty({N}, seg.options().dtype(at::kLong));
+    check_status(txs_ingroup_inds(i32p(seg), opt_i32p(perm), i32p(preSum), N, num_unq,
+                                  N ? out.data_ptr<int64_t>() : nullptr, cur_stream(seg)),
+                 "ingroup_inds");
+    return out;
 }
 
 Tensor make_scratch(int64_t num_special, int64_t C, const Tensor &like) {
@@ -271,6 +354,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("getPreSum", &get_presum_ref, "CSR offsets from a sorted unq_inv (HIP)");
     m.def("build_plan", &build_plan, "build_plan(unq_inv, num_unq, heavy_threshold, unq_cnts|None)");
     m.def("plan_from_presum", &plan_from_presum, "index preparation from CSR offsets");
+    m.def("voxel_keys", &voxel_keys, "voxel_keys(points, range_lo, voxel_size, dims) -> (coors, keys, stats)");
+    m.def("unique_plan", &unique_plan, "unique_plan(keys, key_bound, heavy_threshold, stats|None)");
+    m.def("ingroup_inds", &ingroup_inds, "ingroup_inds(seg, perm|None, preSum, num_unq)");
     m.def("make_scratch", &make_scratch, "zeroed scratch table for the special voxels");
     m.def("forward", &forward, "forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, max_cnt)");
     m.def("backward", &backward, "backward(op, grad_out, arg, perm, seg, preSum, num_total)");

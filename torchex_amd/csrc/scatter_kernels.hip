@@ -325,10 +325,13 @@ __device__ __forceinline__ int wave_max_i32(int x) {
 // would dominate the kernel.
 constexpr int kSpecialThreads = 1024;
 __global__ __launch_bounds__(kSpecialThreads) void plan_special_kernel(
-    const int *__restrict__ preSum, int U, int heavy_threshold,
+    const int *__restrict__ preSum, int U_arg, int heavy_threshold,
     const long long *__restrict__ unq_cnts, int *__restrict__ slot_of,
-    int *__restrict__ heavy_ids, int *__restrict__ stats) {
+    int *__restrict__ heavy_ids, int *__restrict__ stats, const int *__restrict__ num_unq_dev,
+    long long *__restrict__ cnts_out) {
     __shared__ int s_max[kSpecialThreads / 64], s_empty[kSpecialThreads / 64], s_bad[kSpecialThreads / 64];
+    // the voxel count may only be known on the device (unique path): U_arg is then an upper bound
+    const int U = num_unq_dev ? min(U_arg, *num_unq_dev) : U_arg;
     const int u = blockIdx.x * blockDim.x + threadIdx.x;
     const bool in = u < U;
     const int c = in ? preSum[u + 1] - preSum[u] : 0;
@@ -355,6 +358,7 @@ __global__ __launch_bounds__(kSpecialThreads) void plan_special_kernel(
         if (b) stats[TXS_STAT_COUNT_MISMATCH] = 1;
     }
     if (!in) return;
+    if (cnts_out) cnts_out[u] = (long long)c;
     int slot = -1;
     if (c > heavy_threshold || c == 0) {
         slot = atomicAdd(&stats[TXS_STAT_NUM_SPECIAL], 1);
@@ -473,6 +477,91 @@ __global__ void seg_from_presum_kernel(const int *__restrict__ preSum, long n, i
     }
     int flag = (slot_of[lo] >= 0) ? kSpecialBit : 0;
     seg[j] = lo | flag;
+}
+
+// ------------------------------------------------ voxelization front-end --
+
+// torch.div(a, b, rounding_mode='floor') for fp32 (c10::div_floor_floating,
+// c10/util/generic_math.h): Python's floor division, not floor(a / b).
+__device__ __forceinline__ float div_floor_f32(float a, float b) {
+    if (b == 0.0f) return a / b;
+    const float mod = fmodf(a, b);
+    float div = (a - mod) / b;
+    if ((mod != 0.0f) && ((b < 0.0f) != (mod < 0.0f))) div -= 1.0f;
+    float fl;
+    if (div != 0.0f) {
+        fl = floorf(div);
+        if (div - fl > 0.5f) fl += 1.0f;
+    } else {
+        fl = copysignf(0.0f, a / b);
+    }
+    return fl;
+}
+
+// coors = floor((p - lo) / voxel) per axis, key = (x * Y + y) * Z + z
+// (test/test_incremental_mask.py:20-26, operator_py/incremental_points.py:18-19)
+__global__ void voxel_keys_kernel(const float *__restrict__ pts, long n, int stride, float lo0,
+                                  float lo1, float lo2, float v0, float v1, float v2, int d0, int d1,
+                                  int d2, int *__restrict__ coors, int *__restrict__ keys,
+                                  int *__restrict__ stats) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float *p = pts + i * stride;
+    const int x = (int)div_floor_f32(p[0] - lo0, v0);
+    const int y = (int)div_floor_f32(p[1] - lo1, v1);
+    const int z = (int)div_floor_f32(p[2] - lo2, v2);
+    if (coors) {
+        coors[i * 3 + 0] = x;
+        coors[i * 3 + 1] = y;
+        coors[i * 3 + 2] = z;
+    }
+    const bool ok = (unsigned)x < (unsigned)d0 && (unsigned)y < (unsigned)d1 && (unsigned)z < (unsigned)d2;
+    if (!ok) stats[TXS_STAT_OUT_OF_RANGE] = 1;
+    keys[i] = ok ? (x * d1 + y) * d2 + z : 0;
+}
+
+// 1 where a new run of equal keys starts
+__global__ void run_flags_kernel(const int *__restrict__ ks, long n, int *__restrict__ flags) {
+    long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j < n) flags[j] = (j == 0 || ks[j] != ks[j - 1]) ? 1 : 0;
+}
+
+// What torch.unique(keys, return_inverse=True, return_counts=True) returns,
+// from the sorted keys and the exclusive scan `ex` of the run-start flags,
+// plus the plan arrays: run index rid = ex[j] + flag - 1.
+__global__ void unique_finish_kernel(const int *__restrict__ ks, const int *__restrict__ perm,
+                                     const int *__restrict__ ex, long n, int *__restrict__ seg,
+                                     int *__restrict__ inv, int *__restrict__ unq,
+                                     int *__restrict__ preSum, int *__restrict__ stats) {
+    long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    const bool flag = (j == 0 || ks[j] != ks[j - 1]);
+    const int rid = ex[j] + (flag ? 1 : 0) - 1;
+    const int row = stats[TXS_STAT_UNSORTED] ? perm[j] : (int)j;
+    seg[j] = rid;
+    if ((unsigned)row < (unsigned)n) inv[row] = rid;
+    if (flag) {
+        unq[rid] = ks[j];
+        preSum[rid] = (int)j;
+    }
+    if (j == n - 1) {
+        preSum[rid + 1] = (int)n;
+        stats[TXS_STAT_NUM_UNQ] = rid + 1;
+    }
+}
+
+// rank of every element inside its group (operator_py/ingroup_inds_op.py,
+// src/ingroup_inds/ingroup_inds_kernel.cu:17-30): sorted position minus the
+// group's first position; ascending with the element's index, where the
+// reference's atomic counter hands ranks out in arbitrary order.
+__global__ void ingroup_inds_kernel(const int *__restrict__ seg, const int *__restrict__ perm,
+                                    const int *__restrict__ preSum, long n, int U,
+                                    long long *__restrict__ out) {
+    long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    const int u = seg[j] & kIdMask;
+    const int row = perm ? perm[j] : (int)j;
+    if ((unsigned)u < (unsigned)U && (unsigned)row < (unsigned)n) out[row] = (long long)(j - preSum[u]);
 }
 
 // ----------------------------------------------------------------- forward --
@@ -1175,7 +1264,7 @@ int radix_bits(int64_t U) {
 
 extern "C" {
 
-int txs_abi_version(void) { return 3; }
+int txs_abi_version(void) { return 4; }
 
 const char *txs_status_string(int status) {
     switch (status) {
@@ -1266,13 +1355,14 @@ int txs_plan_presum(const int32_t *sorted_keys, int64_t num_total, int64_t num_u
 
 int txs_plan_special(const int32_t *preSum, int64_t num_unq, int32_t heavy_threshold,
                      const int64_t *unq_cnts, int32_t *slot_of, int32_t *heavy_ids, int32_t *stats,
-                     void *stream) {
+                     const int32_t *num_unq_dev, int64_t *cnts_out, void *stream) {
     if (!fits_i32(num_unq) || !preSum || !stats || heavy_threshold < kChunk) return TXS_ERR_INVALID_ARG;
     if (num_unq == 0) return TXS_OK;
     if (!slot_of || !heavy_ids) return TXS_ERR_INVALID_ARG;
     plan_special_kernel<<<dim3(blocks_for(num_unq, kSpecialThreads)), dim3(kSpecialThreads), 0,
                           (hipStream_t)stream>>>(
-        preSum, (int)num_unq, heavy_threshold, (const long long *)unq_cnts, slot_of, heavy_ids, stats);
+        preSum, (int)num_unq, heavy_threshold, (const long long *)unq_cnts, slot_of, heavy_ids, stats,
+        num_unq_dev, (long long *)cnts_out);
     return status_of(hipGetLastError());
 }
 
@@ -1293,6 +1383,53 @@ int txs_plan_seg_from_presum(const int32_t *preSum, int64_t num_total, int64_t n
     if (!preSum || !slot_of || !seg || num_unq <= 0) return TXS_ERR_INVALID_ARG;
     seg_from_presum_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
         preSum, num_total, (int)num_unq, slot_of, seg);
+    return status_of(hipGetLastError());
+}
+
+int txs_voxel_keys(const float *points, int64_t num_total, int64_t point_stride,
+                   const float *range_lo, const float *voxel_size, const int32_t *dims,
+                   int32_t *coors, int32_t *keys, int32_t *stats, void *stream) {
+    if (!fits_i32(num_total) || point_stride < 3 || !range_lo || !voxel_size || !dims || !stats)
+        return TXS_ERR_INVALID_ARG;
+    const long long cells = (long long)dims[0] * dims[1] * dims[2];
+    if (dims[0] <= 0 || dims[1] <= 0 || dims[2] <= 0 || !fits_i32(cells)) return TXS_ERR_INVALID_ARG;
+    if (num_total == 0) return TXS_OK;
+    if (!points || !keys) return TXS_ERR_INVALID_ARG;
+    voxel_keys_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+        points, num_total, (int)point_stride, range_lo[0], range_lo[1], range_lo[2], voxel_size[0],
+        voxel_size[1], voxel_size[2], dims[0], dims[1], dims[2], coors, keys, stats);
+    return status_of(hipGetLastError());
+}
+
+int64_t txs_unique_workspace_len(int64_t num_total) { return num_total + scan_tiles(num_total + 1) + 17; }
+
+int txs_unique_runs(const int32_t *sorted_keys, const int32_t *perm, int64_t num_total,
+                    int32_t *unique_ws, int32_t *seg, int32_t *unq_inv, int32_t *unq_keys,
+                    int32_t *preSum, int32_t *stats, void *stream) {
+    if (!fits_i32(num_total) || !stats || !preSum) return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    if (num_total == 0) {
+        fill_i32_kernel<<<dim3(1), dim3(64), 0, st>>>(preSum, 1, 0);
+        return status_of(hipGetLastError());
+    }
+    if (!sorted_keys || !perm || !unique_ws || !seg || !unq_inv || !unq_keys) return TXS_ERR_INVALID_ARG;
+    const long n = num_total;
+    int *flags = unique_ws;
+    int *scan_ws = unique_ws + n;
+    run_flags_kernel<<<dim3(blocks_for(n)), dim3(kThreads), 0, st>>>(sorted_keys, n, flags);
+    if (exclusive_scan(flags, n, flags, n, scan_ws, st) != hipSuccess) return TXS_ERR_LAUNCH;
+    unique_finish_kernel<<<dim3(blocks_for(n)), dim3(kThreads), 0, st>>>(sorted_keys, perm, flags, n, seg,
+                                                                       unq_inv, unq_keys, preSum, stats);
+    return status_of(hipGetLastError());
+}
+
+int txs_ingroup_inds(const int32_t *seg, const int32_t *perm, const int32_t *preSum,
+                     int64_t num_total, int64_t num_unq, int64_t *out, void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_unq)) return TXS_ERR_INVALID_ARG;
+    if (num_total == 0) return TXS_OK;
+    if (!seg || !preSum || !out || num_unq <= 0) return TXS_ERR_INVALID_ARG;
+    ingroup_inds_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+        seg, perm, preSum, num_total, (int)num_unq, (long long *)out);
     return status_of(hipGetLastError());
 }
 

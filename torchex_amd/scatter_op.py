@@ -68,6 +68,48 @@ class ScatterData:
         self.num_unq = num_unq
         self._scratch = {}
 
+    @classmethod
+    def from_keys(cls, keys, key_bound, heavy_threshold=None, max_tie_rule="first", _stats=None):
+        """ScatterData straight from voxel keys (any non-negative int ids below
+        ``key_bound``, e.g. linear voxel ids): computes what ``torch.unique(keys,
+        return_inverse=True, return_counts=True)`` returns -- kept as ``unq_keys``,
+        ``unq_inv``, ``unq_cnts`` -- and the scatter plan from ONE sort of the keys,
+        where ``torch.unique`` followed by ``ScatterData(...)`` sorts twice."""
+        if max_tie_rule not in ("first", "reference"):
+            raise ValueError("max_tie_rule must be 'first' or 'reference'")
+        self = cls.__new__(cls)
+        self.max_tie_rule = max_tie_rule
+        if heavy_threshold is None:
+            heavy_threshold = scatter_ext.default_heavy_threshold()
+        self.heavy_threshold = int(heavy_threshold)
+        flat = keys.reshape(-1)
+        if flat.dtype != torch.int32:
+            flat = flat.int()
+        flat = flat.contiguous()
+        (self.unq_keys, self.unq_inv, cnts, self.preSum, self.perm, self.seg, self.slot_of,
+         self.heavy_ids, stats) = scatter_ext.unique_plan(flat, int(key_bound), self.heavy_threshold, _stats)
+        self.unq_cnts = cnts.unsqueeze(-1)
+        self.num_total = flat.shape[0]
+        self.is_sorted = self.perm is None
+        self.max_cnt = int(stats[2])
+        self.num_special = int(stats[3])
+        self.num_unq = int(stats[6])
+        self._scratch = {}
+        return self
+
+    @classmethod
+    def from_points(cls, points, voxel_size, pc_range, heavy_threshold=None, max_tie_rule="first"):
+        """Dynamic voxelization in one go: voxel coordinates as the reference's
+        ``voxelize_single`` computes them (``test/test_incremental_mask.py:20-26``),
+        x-major linear keys (``operator_py/incremental_points.py:18-19``), unique and
+        scatter plan.  Points outside ``pc_range`` raise.  Extra attributes:
+        ``coors`` (int32 ``[N, 3]``), ``spatial_size``."""
+        coors, keys, stats, dims = _voxel_keys(points, voxel_size, pc_range)
+        self = cls.from_keys(keys, dims[0] * dims[1] * dims[2], heavy_threshold, max_tie_rule, _stats=stats)
+        self.coors = coors
+        self.spatial_size = dims
+        return self
+
     def scratch(self, channel):
         """Zeroed table the special voxels are merged in; the kernels leave it
         zeroed again, so one buffer per channel count is kept for reuse."""
@@ -178,6 +220,39 @@ class GetPreSumFunction(Function):
     @staticmethod
     def backward(ctx, g):
         return None
+
+
+def _voxel_keys(points, voxel_size, pc_range):
+    import math
+    lo = [float(v) for v in pc_range[:3]]
+    hi = [float(v) for v in pc_range[3:6]]
+    vs = [float(v) for v in voxel_size]
+    dims = [max(1, int(math.ceil((h - l) / v - 1e-6))) for l, h, v in zip(lo, hi, vs)]
+    coors, keys, stats = scatter_ext.voxel_keys(points, lo, vs, dims)
+    return coors, keys, stats, dims
+
+
+def voxelize(points, voxel_size, pc_range):
+    """Voxel coordinates of every point: ``torch.div(points[:, :3] - pc_range[:3],
+    voxel_size, rounding_mode='floor').int()`` (the reference's ``voxelize_single``,
+    ``test/test_incremental_mask.py:20-26``), int32 ``[N, 3]``, computed by one HIP
+    kernel.  No range check is made here (as in the reference)."""
+    return _voxel_keys(points, voxel_size, pc_range)[0]
+
+
+def ingroup_inds(group_inds):
+    """Rank of every element inside its group (``operator_py/ingroup_inds_op.py``).
+    ``group_inds``: integer ``[N]`` group ids; returns ``[N]`` of the same dtype.
+    Ranks ascend with the element index inside a group; the reference hands
+    them out with an atomic counter, i.e. in arbitrary order."""
+    ids = group_inds.reshape(-1)
+    if ids.numel() == 0:
+        return torch.zeros_like(group_inds)
+    num_groups = int(ids.max()) + 1          # the reference reads the max on the host too
+    ids32 = ids.int().contiguous()
+    preSum, perm, seg, _, _, _ = scatter_ext.build_plan(ids32, num_groups, scatter_ext.default_heavy_threshold(), None)
+    out = scatter_ext.ingroup_inds(seg, perm, preSum, num_groups)
+    return out.to(group_inds.dtype).reshape(group_inds.shape)
 
 
 scatter_sum = ScatterSumFunction.apply
