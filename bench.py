@@ -120,6 +120,38 @@ def main():
     torch.cuda.synchronize()
     prep_ms = (time.perf_counter() - t0) / 5 * 1e3
 
+    # front-end: keys -> (unique, inverse, counts) + plan.  torch.unique followed by
+    # ScatterData sorts twice; ScatterData.from_keys sorts once.
+    keys_cpu, key_bound = workloads._lidar_keys(N, torch.Generator().manual_seed(2))
+    keys = keys_cpu.to(dev)
+
+    def wall_ms(fn, iters=5):
+        fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / iters * 1e3
+
+    def torch_unique_then_plan():
+        _, i2, c2 = torch.unique(keys, return_inverse=True, return_counts=True)
+        return T.ScatterData(i2, c2)
+
+    frontend = {
+        "torch_unique_plus_ScatterData_ms": wall_ms(torch_unique_then_plan),
+        "ScatterData_from_keys_ms": wall_ms(lambda: T.ScatterData.from_keys(keys, key_bound)),
+    }
+    pts = (torch.rand((N, 4), generator=torch.Generator().manual_seed(5)) * 150.0 - 75.0).to(dev)
+    pts[:, 2] = pts[:, 2] * (6.0 / 150.0) + 1.0
+    vs_t = torch.tensor([0.2, 0.2, 0.2], device=dev)
+    lo_t = torch.tensor([-75.0, -75.0, -2.0], device=dev)
+    frontend["voxelize_ms"] = wall_ms(lambda: T.voxelize(pts, [0.2, 0.2, 0.2], [-75, -75, -2, 75, 75, 4]), 20)
+    frontend["torch_div_floor_voxelize_ms"] = wall_ms(
+        lambda: torch.div(pts[:, :3] - lo_t[None, :], vs_t[None, :], rounding_mode="floor").int(), 20)
+    frontend["ScatterData_from_points_ms"] = wall_ms(
+        lambda: T.ScatterData.from_points(pts, [0.2, 0.2, 0.2], [-75, -75, -2, 75, 75, 4]))
+
     def step():
         feats.grad = None
         T.scatter_mean(feats, data).backward(g_mean)
@@ -191,6 +223,8 @@ def main():
         "per_kernel": per_kernel,
         "device_copy_GBps": copy_gbps,
         "index_prep_ms": prep_ms,
+        "step_incl_index_prep_ms": ms_per_step + prep_ms,
+        "frontend": frontend,
     }
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, g_mean_cpu, g_max_cpu)
