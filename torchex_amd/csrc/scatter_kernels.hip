@@ -1027,8 +1027,11 @@ __global__ __launch_bounds__(kThreads) void scatter_bwd_kernel(
             if (ll == la || seg_s[ll - 1] != u) {
                 bt.need |= 1u << i;
                 const size_t o = (size_t)u * C + col;
+                // upstream rows are re-read by the neighbouring chunk when a run
+                // straddles it (keep them cached); an arg row is consumed here and
+                // nowhere else (stream it)
                 bt.gv[i] = ld<raw, VEC>(g + o);
-                if (OP == TXS_MAX) bt.av[i] = ld<int, VEC>(arg + o);
+                if (OP == TXS_MAX) bt.av[i] = ld_stream<int, VEC>(arg + o);
                 if (OP == TXS_MEAN) bt.cnt[i] = preSum[u + 1] - preSum[u];
             }
         }
