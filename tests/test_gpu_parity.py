@@ -558,3 +558,85 @@ def test_reference_tie_rule_mode_matches_default_without_ties():
     a = T.scatter_max(f, T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV)))
     b = T.scatter_max(f, T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV), max_tie_rule="reference"))
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+# ------------------------------------------------------------ robustness ----
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("C", [1, 2, 8, 13, 16, 72])
+def test_half_precision_channel_widths(C, dtype):
+    g = torch.Generator().manual_seed(100 + C)
+    N, U = 4000, 61
+    inv = torch.randint(0, U, (N,), generator=g)
+    inv[:U] = torch.arange(U)
+    run_case(f"half_channels{C}", torch.randn((N, C), generator=g), inv, torch.bincount(inv, minlength=U),
+             dtype=dtype)
+
+
+def test_many_rows_few_channels():
+    """Index range and tile geometry at the other extreme: 12M rows of 2 channels (one lane per
+    row, 4096 positions per workgroup)."""
+    T = tx()
+    g = torch.Generator().manual_seed(77)
+    N, U, C = 12_000_000, 900_000, 2
+    inv = torch.randint(0, U, (N,), generator=g)
+    feats = torch.randint(-50, 51, (N, C), generator=g).float()      # exact sums
+    cnts = torch.bincount(inv, minlength=U)
+    say(f"[case] many rows N={N} C={C} U={U}")
+    data = T.ScatterData(inv.to(DEV), cnts.to(DEV))
+    f = feats.to(DEV)
+    s = T.scatter_sum(f, data).cpu()
+    want = torch.zeros((U, C)).index_add_(0, inv, feats)
+    assert torch.equal(s, want)
+    mx, arg = T.scatter_max(f, data)
+    wm, wa = orc.scatter_max_first(feats.numpy(), inv.numpy().astype(np.int32), U)
+    assert np.array_equal(arg.cpu().numpy(), wa) and bits_equal(mx.cpu().numpy(), wm)
+    gup = torch.randint(-5, 6, (U, C), generator=g).float().to(DEV)
+    x = f.clone().requires_grad_(True)
+    T.scatter_sum(x, data).backward(gup)
+    assert torch.equal(x.grad, gup[inv.to(DEV)])
+
+
+def test_misaligned_views_fall_back_to_narrow_vectors():
+    """Tensors whose storage offset breaks 16-byte alignment still work (the launcher picks a
+    narrower per-lane vector)."""
+    T = tx()
+    import scatter_ext
+    g = torch.Generator().manual_seed(88)
+    N, U, C = 5000, 123, 128
+    inv = torch.randint(0, U, (N,), generator=g)
+    inv[:U] = torch.arange(U)
+    feats = torch.randn((N, C), generator=g)
+    data = T.ScatterData(inv.to(DEV), torch.bincount(inv, minlength=U).to(DEV))
+    base = torch.empty(N * C + 3, device=DEV)
+    for off in (1, 2, 3):
+        f = base[off:off + N * C].view(N, C)
+        f.copy_(feats)
+        assert f.data_ptr() % 16 != 0 and f.is_contiguous()
+        say(f"[case] misaligned feats offset {off} floats")
+        mx, arg = T.scatter_max(f, data)
+        wm, wa = orc.scatter_max_first(feats.numpy(), inv.numpy().astype(np.int32), U)
+        assert np.array_equal(arg.cpu().numpy(), wa) and bits_equal(mx.cpu().numpy(), wm)
+        gbase = torch.empty(U * C + 3, device=DEV)
+        gup = gbase[off:off + U * C].view(U, C)
+        gup.copy_(workloads.upstream_grad(U, C, 5))
+        gin = scatter_ext.backward(scatter_ext.MAX, gup, arg, data.perm, data.seg, data.preSum, N)
+        assert bits_equal(gin.cpu().numpy(), orc.max_backward(gup.cpu().numpy(), wa, N))
+
+
+def test_runs_on_the_current_stream():
+    T = tx()
+    w = workloads.lidar_sweep(N=200_000, C=64, seed=21)
+    inv, cnts, f = w.unq_inv.to(DEV), w.unq_cnts.to(DEV), w.feats.to(DEV)
+    ref = T.scatter_max(f, T.ScatterData(inv, cnts))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        data = T.ScatterData(inv, cnts)
+        outs = [T.scatter_max(f, data) for _ in range(3)]
+        means = [T.scatter_mean(f, data) for _ in range(3)]
+    side.synchronize()
+    for mx, arg in outs:
+        assert torch.equal(mx, ref[0]) and torch.equal(arg, ref[1])
+    light = (w.unq_cnts <= data.heavy_threshold).to(DEV)
+    assert torch.equal(means[0][light], means[2][light])
