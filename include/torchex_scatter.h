@@ -164,6 +164,38 @@ int64_t txs_unique_workspace_len(int64_t num_total);
 int txs_ingroup_inds(const int32_t *seg, const int32_t *perm, const int32_t *preSum,
                      int64_t num_total, int64_t num_unq, int64_t *out, void *stream);
 
+/* Points inside (enlarged) rotated boxes.  Replaces dynamic_point_pool_launcher
+ * (torchex/src/dynamic_point_pool/dynamic_point_pool.cpp:20-32, kernels
+ * dynamic_point_pool_kernel.cu:73-170,280-310): for every (box, point) pair with
+ * the point inside the box enlarged by extra_wlh (HOST array of 3), one output
+ * entry: point index, box index and 13 floats (x, y, z, local x/y/z, the six
+ * face offsets, in-margin flag).  At most max_pts_per_box entries per box and
+ * max_all_pts in total.  Entries are written compactly at [0, *num_out) in
+ * (box, point) order -- deterministic, where the reference's atomic counters
+ * give an arbitrary order and an arbitrary surviving subset under the caps.
+ * rois [num_boxes, 7] (x, y, z of the bottom centre, w, l, h, rz), pts
+ * [num_pts, 3]; outputs are caller-allocated with max_all_pts entries and
+ * need no initialisation; num_out is a device int.  workspace: int32 array of
+ * txs_dpp_workspace_len(num_pts, num_boxes) entries, 8-byte aligned. */
+int txs_dynamic_point_pool(const float *rois, const float *pts, int64_t num_boxes, int64_t num_pts,
+                           const float *extra_wlh, int32_t max_pts_per_box, int64_t max_all_pts,
+                           int32_t *workspace, int64_t *out_pts_idx, int64_t *out_roi_idx,
+                           float *out_pts_feats, int32_t *num_out, void *stream);
+int64_t txs_dpp_workspace_len(int64_t num_pts, int64_t num_boxes);
+
+/* Hash table of int32 (key, value) pairs.  Replace build_hash_table_launcher /
+ * probe_hash_table_launcher (torchex/src/grid_hash/grid_hash.cpp:14-27, kernels
+ * grid_hash_kernel.cu:19-49, probing of src/utils/functions.cuh:30-64).
+ * table: int32 [table_size, 2], table_size a power of two >= num_keys, 8-byte
+ * aligned; build fills it with -1 first.  Keys must be unique and >= 0.
+ * fail_flag (may be NULL): device int set to 1 if a key could not be placed.
+ * probe writes the value of each key, or -1 for a key that is not in the table
+ * (the reference asserts instead). */
+int txs_grid_hash_build(const int32_t *keys, const int32_t *values, int64_t num_keys, int32_t *table,
+                        int64_t table_size, int32_t *fail_flag, void *stream);
+int txs_grid_hash_probe(const int32_t *keys, int64_t num_keys, const int32_t *table,
+                        int64_t table_size, int32_t *out_values, void *stream);
+
 /* ---- the hot path --------------------------------------------------------- */
 
 /* Forward reduction.  Replaces scatter_sum_launcher / scatter_max_launcher

@@ -211,3 +211,37 @@ def voxelize(points, voxel_size, range_lo, dims):
     keys = np.empty(n, dtype=np.int32)
     lib().orc_voxelize(_p(pts), _ll(n), _ll(pts.shape[1]), _p(lo), _p(vs), _p(dm), _p(coors), _p(keys))
     return coors, keys
+
+
+def dynamic_point_pool(rois, pts, extra_wlh, max_pts, max_all):
+    r = _f32(rois)
+    p = _f32(pts)
+    e = _f32(extra_wlh)
+    idx = np.full(max_all, -1, dtype=np.int64)
+    roi = np.full(max_all, -1, dtype=np.int64)
+    feats = np.zeros((max_all, 13), dtype=np.float32)
+    lib().orc_dynamic_point_pool.restype = ctypes.c_int64
+    m = lib().orc_dynamic_point_pool(_p(r), _ll(r.shape[0]), _p(p), _ll(p.shape[0]), _p(e),
+                                     ctypes.c_int(int(max_pts)), _ll(max_all), _p(idx), _p(roi), _p(feats))
+    return idx[:m], roi[:m], feats[:m]
+
+
+def grid_hash_build(keys, values):
+    k = _i32(keys)
+    v = _i32(values)
+    size = 1
+    while size < max(k.shape[0], 1):
+        size <<= 1
+    table = np.full((size, 2), -1, dtype=np.int32)
+    rc = lib().orc_grid_hash_build(_p(k), _p(v), _ll(k.shape[0]), _p(table), ctypes.c_int(size))
+    if rc != 0:
+        raise RuntimeError("hash table full")
+    return table
+
+
+def grid_hash_probe(keys, table):
+    k = _i32(keys)
+    t = _i32(table)
+    out = np.empty(k.shape[0], dtype=np.int32)
+    lib().orc_grid_hash_probe(_p(k), _ll(k.shape[0]), _p(t), ctypes.c_int(t.shape[0]), _p(out))
+    return out

@@ -386,3 +386,97 @@ void orc_voxelize(const float *points, int64_t n, int64_t stride, const float *l
         keys[i] = (c[0] * dims[1] + c[1]) * dims[2] + c[2];
     }
 }
+
+/* ---- dynamic point pool -------------------------------------------------
+ * torchex/src/dynamic_point_pool/dynamic_point_pool_kernel.cu:22-170 (test and
+ * 13 numbers per hit) and :280-310 (compaction), with the two atomic counters
+ * (:108-113) advanced in (box, point) order -- the order the reference's own
+ * wrapper comment calls the usual one.  Mixed float/double arithmetic as
+ * written there; the rotation terms cos/sin(rz + pi/2) are evaluated in double
+ * and rounded to float (the device's cosf/sinf is within an ulp of that).
+ * Returns the number of entries written. */
+int64_t orc_dynamic_point_pool(const float *rois, int64_t B, const float *pts, int64_t P,
+                               const float *extra_wlh, int max_pts, int64_t max_all,
+                               int64_t *out_pts_idx, int64_t *out_roi_idx, float *out_feats) {
+    int64_t global = 0;
+    for (int64_t b = 0; b < B; ++b) {
+        const float *r = rois + b * 7;
+        const float cx = r[0], cy = r[1], w = r[3], l = r[4], h = r[5];
+        const float large_w = w + extra_wlh[0], large_l = l + extra_wlh[1], large_h = h + extra_wlh[2];
+        const float cz = (float)((double)r[2] + (double)h / 2.0);
+        const float rot = (float)((double)r[6] + 3.14159265358979323846 / 2); /* M_PI / 2 */
+        const float cosa = (float)cos((double)rot), sina = (float)sin((double)rot);
+        int in_box_counter = 0;
+        for (int64_t p = 0; p < P; ++p) {
+            const float x = pts[p * 3], y = pts[p * 3 + 1], z = pts[p * 3 + 2];
+            if ((double)fabsf(z - cz) > (double)large_h / 2.0) continue;
+            volatile float sx = x - cx, sy = y - cy;
+            volatile float t1 = sx * cosa, t2 = sy * (-sina), t3 = sx * sina, t4 = sy * cosa;
+            volatile float local_x = t1 + t2, local_y = t3 + t4;
+            const double lx = local_x, ly = local_y;
+            const int in_flag = (lx > -(double)l / 2.0) & (lx < (double)l / 2.0) & (ly > -(double)w / 2.0) &
+                                (ly < (double)w / 2.0) & ((double)fabsf(z - cz) < (double)h / 2.0);
+            const int in_large = (lx > -(double)large_l / 2.0) & (lx < (double)large_l / 2.0) &
+                                 (ly > -(double)large_w / 2.0) & (ly < (double)large_w / 2.0);
+            const int flag = in_flag ? 2 : (in_large ? 1 : 0);
+            if (!flag) continue;
+            const int cnt = in_box_counter++;
+            if (cnt >= max_pts) continue;
+            const int64_t pos = global++;
+            if (pos >= max_all) continue;
+            volatile float local_z = (float)((double)z - ((double)r[2] + (double)h / 2.0));
+            float *f = out_feats + pos * 13;
+            out_pts_idx[pos] = p;
+            out_roi_idx[pos] = b;
+            f[0] = x; f[1] = y; f[2] = z;
+            f[3] = local_x; f[4] = local_y; f[5] = local_z;
+            { volatile float v = local_x + l / 2; f[6] = v; }
+            { volatile float v = local_y + w / 2; f[7] = v; }
+            { volatile float v = local_z + h / 2; f[8] = v; }
+            { volatile float v = -local_x + l / 2; f[9] = v; }
+            { volatile float v = -local_y + w / 2; f[10] = v; }
+            { volatile float v = -local_z + h / 2; f[11] = v; }
+            f[12] = flag == 1 ? 1.0f : 0.0f;
+        }
+    }
+    return global < max_all ? global : max_all;
+}
+
+/* ---- grid hash ------------------------------------------------------------
+ * torchex/src/utils/functions.cuh:30-64 with the inserts applied in index
+ * order.  table: int32 [table_size, 2], filled with -1 by the caller. */
+static int orc_double_hash(long long key, int probe_i, int table_size) {
+    return (int)((key % table_size + probe_i * (key * 2 + 1)) % table_size);
+}
+int orc_grid_hash_build(const int32_t *keys, const int32_t *values, int64_t n, int32_t *table,
+                        int table_size) {
+    for (int64_t k = 0; k < n; ++k) {
+        int placed = 0;
+        for (int i = 0; i < table_size && !placed; ++i) {
+            const int s = orc_double_hash(keys[k], i, table_size);
+            if (table[2 * s] == -1) {
+                table[2 * s] = keys[k];
+                table[2 * s + 1] = values[k];
+                placed = 1;
+            }
+        }
+        if (!placed) return -1;
+    }
+    return 0;
+}
+void orc_grid_hash_probe(const int32_t *keys, int64_t n, const int32_t *table, int table_size,
+                         int32_t *out) {
+    for (int64_t k = 0; k < n; ++k) {
+        out[k] = -1;
+        for (int i = 0; i < table_size; ++i) {
+            const int s = orc_double_hash(keys[k], i, table_size);
+            if (table[2 * s] == keys[k]) {
+                out[k] = table[2 * s + 1];
+                break;
+            }
+            /* functions.cuh:54-63 scans all table_size slots before returning -1;
+             * an empty slot already proves absence (no deletions), same answer */
+            if (table[2 * s] == -1) break;
+        }
+    }
+}

@@ -147,3 +147,123 @@ def test_ingroup_inds():
     s = torch.sort(ids).values.int()
     assert T.ingroup_inds(s.to(DEV)).dtype == torch.int32
     assert np.array_equal(T.ingroup_inds(s.to(DEV)).cpu().numpy(), orc.ingroup_inds(s.numpy()).astype(np.int32))
+
+
+# ---------------------------------------------------------- dynamic point pool --
+
+def _boxes_and_points(seed, B, P):
+    g = torch.Generator().manual_seed(seed)
+    rois = torch.zeros((B, 7))
+    rois[:, 0:2] = torch.rand((B, 2), generator=g) * 100 - 50
+    rois[:, 2] = torch.rand((B,), generator=g) * 2 - 1
+    rois[:, 3:6] = torch.rand((B, 3), generator=g) * 4 + 1
+    rois[:, 6] = torch.rand((B,), generator=g) * 6.283 - 3.1415
+    pts = torch.zeros((P, 3))
+    pts[:, 0:2] = torch.rand((P, 2), generator=g) * 120 - 60
+    pts[:, 2] = torch.rand((P,), generator=g) * 6 - 2
+    per = P // (2 * B)
+    for b in range(B):
+        pts[b * per:(b + 1) * per, 0:2] = rois[b, 0:2] + (torch.rand((per, 2), generator=g) - 0.5) * 7
+        pts[b * per:(b + 1) * per, 2] = rois[b, 2] + torch.rand((per,), generator=g) * rois[b, 5]
+    return rois, pts[torch.randperm(P, generator=g)]
+
+
+@pytest.mark.parametrize("B,P,cap,max_all,extra", [
+    (40, 60_000, 512, 50_000, [0.0, 0.0, 0.0]),      # the reference test's call: dynamic_point_pool(boxes, pc, [0,0,0], 512)
+    (40, 60_000, 100_000, 1_000_000, [0.5, 0.5, 0.3]),
+    (7, 1_000, 16, 60, [1.0, 0.2, 0.4]),             # both caps bite
+    (300, 200_000, 64, 50_000, [0.4, 0.4, 0.2]),
+    (1, 300, 512, 50_000, [0.0, 0.0, 0.0]),
+])
+def test_dynamic_point_pool(B, P, cap, max_all, extra):
+    """Bit-exact against the oracle: same hits, same (box, point) order, same 13 floats
+    (both sides take the rotation terms from double-precision cos/sin and keep products
+    and sums as separate fp32 roundings)."""
+    T = tx()
+    rois, pts = _boxes_and_points(B * 7 + P, B, P)
+    say(f"[case] dynamic_point_pool B={B} P={P} cap={cap} max_all={max_all}")
+    idx, roi, feats = T.dynamic_point_pool(rois.to(DEV), pts.to(DEV), extra, cap, max_all)
+    wi, wr, wf = orc.dynamic_point_pool(rois.numpy(), pts.numpy(), extra, cap, max_all)
+    assert idx.dtype == torch.int64 and roi.dtype == torch.int64 and feats.shape[1] == 13
+    assert wi.shape[0] > 0
+    assert np.array_equal(idx.cpu().numpy(), wi) and np.array_equal(roi.cpu().numpy(), wr)
+    assert np.array_equal(feats.cpu().numpy().view(np.uint32), wf.view(np.uint32))
+    assert idx.shape[0] <= max_all and torch.bincount(roi).max().item() <= cap
+
+
+def test_dynamic_point_pool_no_hits_returns_the_reference_placeholder():
+    T = tx()
+    rois = torch.tensor([[1000.0, 1000.0, 0.0, 2.0, 4.0, 1.5, 0.3]], device=DEV)
+    pts = torch.rand((500, 3), device=DEV)
+    idx, roi, feats = T.dynamic_point_pool(rois, pts, [0, 0, 0], 512)
+    assert idx.tolist() == [-1] and roi.tolist() == [-1] and feats.shape == (1, 13) and (feats == 0).all()
+    with pytest.raises(RuntimeError):
+        T.dynamic_point_pool(rois.cpu(), pts, [0, 0, 0], 512)
+
+
+def test_dynamic_point_pool_feeds_the_scatter_path():
+    """The pairs this op emits are what FSD-style code then reduces per RoI: unique the
+    roi ids and scatter the per-pair numbers (here through ScatterData.from_keys)."""
+    T = tx()
+    rois, pts = _boxes_and_points(99, 50, 80_000)
+    idx, roi, feats = T.dynamic_point_pool(rois.to(DEV), pts.to(DEV), [0.3, 0.3, 0.2], 512, 200_000)
+    data = T.ScatterData.from_keys(roi, 50)
+    assert data.is_sorted                               # (box, point) order: no permutation needed
+    mx, arg = T.scatter_max(feats.contiguous(), data)
+    unq, inv = torch.unique(roi.cpu(), return_inverse=True)
+    wm, wa = orc.scatter_max_first(feats.cpu().numpy(), inv.numpy().astype(np.int32), unq.shape[0])
+    assert np.array_equal(arg.cpu().numpy(), wa) and np.array_equal(mx.cpu().numpy(), wm)
+
+
+# -------------------------------------------------------------------- grid hash --
+
+def test_grid_hash_build_and_probe_against_oracle():
+    T = tx()
+    rng = np.random.default_rng(17)
+    for n in (1, 2, 1000, 1024, 4097, 300_000):
+        keys = rng.choice(2 ** 30, size=n, replace=False).astype(np.int32)
+        vals = rng.permutation(n).astype(np.int32)
+        say(f"[case] grid_hash n={n}")
+        table = T.grid_hash_build(torch.from_numpy(keys).to(DEV), torch.from_numpy(vals).to(DEV))
+        assert table.dtype == torch.int32 and table.shape == (orc.grid_hash_build(keys, vals).shape[0], 2)
+        tb = table.cpu().numpy()
+        stored = tb[tb[:, 0] != -1]
+        assert stored.shape[0] == n and (tb[tb[:, 0] == -1, 1] == -1).all()
+        assert set(map(tuple, stored.tolist())) == set(zip(keys.tolist(), vals.tolist()))
+        # absent keys too; few of them when the table is completely full (n a power of two),
+        # where an absent key has to visit every slot
+        n_absent = 8 if (n & (n - 1)) == 0 else n + 5
+        queries = np.concatenate([keys, rng.integers(0, 2 ** 30, size=n_absent).astype(np.int32)])
+        out = T.grid_hash_probe(torch.from_numpy(queries).to(DEV), table).cpu().numpy()
+        # the table built in a different insertion order answers every query identically
+        assert np.array_equal(out, orc.grid_hash_probe(queries, orc.grid_hash_build(keys, vals)))
+        # and the oracle's probe reads the GPU-built table the same way (open-addressing invariant)
+        assert np.array_equal(orc.grid_hash_probe(queries, tb), out)
+
+
+def test_grid_hash_class_follows_the_reference_test():
+    """test/test_grid_hash.py:17-44 (smaller, seeded): probe(unique rows) == arange, the
+    table maps its own keys to their values, and the mapping is stable under re-indexing."""
+    T = tx()
+    import random
+    random.seed(2)
+    g = torch.Generator().manual_seed(0)
+    for _ in range(6):
+        all_size = random.randint(1, 200000)
+        high = random.randint(10, 1024)
+        coors = torch.randint(0, high, (all_size, 3), generator=g).int()
+        unq_coors = torch.unique(coors, dim=0)
+        hasher = T.GridHash(coors.to(DEV), debug=True)
+        out = hasher.probe(unq_coors.to(DEV))
+        assert (out.cpu() == torch.arange(len(out))).all()
+        valid_values = hasher.valid_table[:, 1]
+        assert (hasher.probe(hasher.table[hasher.valid_mask, 0]) == valid_values).all()
+        index = torch.randint(0, max(all_size - 1, 1), (random.randint(1, 200000),), generator=g)
+        values_1 = hasher.probe(coors.to(DEV))
+        values_2 = hasher.probe(coors[index].to(DEV))
+        assert (values_1[index.to(DEV)] == values_2).all()
+    # flat keys
+    keys = torch.randint(0, 5000, (20000,), generator=g)
+    h = T.GridHash(keys.to(DEV))
+    unq, inv = torch.unique(keys, return_inverse=True)
+    assert torch.equal(h.probe(keys.to(DEV)).cpu().long(), inv)

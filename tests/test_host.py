@@ -31,7 +31,7 @@ def test_header_symbols_are_exported():
 
 def test_host_only_entry_points():
     lib = _lib()
-    assert lib.txs_abi_version() == 4
+    assert lib.txs_abi_version() == 5
     lib.txs_status_string.restype = ctypes.c_char_p
     assert lib.txs_status_string(0) == b"ok"
     assert b"invalid" in lib.txs_status_string(1)

@@ -378,3 +378,89 @@ def test_voxelize_oracle_against_torch_floor_division():
     for a, b in [(7.0, 2.0), (-7.0, 2.0), (7.0, -2.0), (0.3, 0.1), (-0.3, 0.1), (1.0, 0.1)]:
         c, _ = orc.voxelize(np.array([[a, 0, 0]], np.float32), [b, 1, 1], [0, 0, 0], [1 << 20, 1, 1])
         assert c[0, 0] == int(np.float32(a) // np.float32(b)), (a, b)
+
+
+def _boxes_and_points(seed, B=12, P=4000):
+    g = torch.Generator().manual_seed(seed)
+    rois = torch.zeros((B, 7))
+    rois[:, 0:2] = torch.rand((B, 2), generator=g) * 40 - 20
+    rois[:, 2] = torch.rand((B,), generator=g) * 2 - 1
+    rois[:, 3:6] = torch.rand((B, 3), generator=g) * 4 + 1
+    rois[:, 6] = torch.rand((B,), generator=g) * 6.283 - 3.1415
+    pts = torch.zeros((P, 3))
+    pts[:, 0:2] = torch.rand((P, 2), generator=g) * 50 - 25
+    pts[:, 2] = torch.rand((P,), generator=g) * 6 - 2
+    # plant points around every box so that each has hits
+    per = P // (2 * B)
+    for b in range(B):
+        pts[b * per:(b + 1) * per, 0:2] = rois[b, 0:2] + (torch.rand((per, 2), generator=g) - 0.5) * 6
+        pts[b * per:(b + 1) * per, 2] = rois[b, 2] + torch.rand((per,), generator=g) * rois[b, 5]
+    return rois, pts
+
+
+def test_dynamic_point_pool_oracle_geometry():
+    """Pins the restated box test against an independent formulation: rotate the point
+    into the box frame with a rotation matrix in float64 and compare the in-box /
+    in-margin classification and the 13 numbers (float tolerance: the formulas differ
+    in rounding, not in meaning)."""
+    rois, pts = _boxes_and_points(3)
+    extra = [0.6, 0.4, 0.2]
+    idx, roi, feats = orc.dynamic_point_pool(rois.numpy(), pts.numpy(), extra, 10 ** 6, 10 ** 6)
+    assert idx.shape[0] > 500
+    R, Pn = rois.double().numpy(), pts.double().numpy()
+    want = []
+    for b in range(R.shape[0]):
+        cx, cy, cz, w, l, h, rz = R[b]
+        a = rz + np.pi / 2
+        dx, dy, dz = Pn[:, 0] - cx, Pn[:, 1] - cy, Pn[:, 2] - (cz + h / 2)
+        lx = dx * np.cos(a) - dy * np.sin(a)
+        ly = dx * np.sin(a) + dy * np.cos(a)
+        inside = (np.abs(lx) < l / 2) & (np.abs(ly) < w / 2) & (np.abs(dz) < h / 2)
+        large = (np.abs(lx) < (l + extra[1]) / 2) & (np.abs(ly) < (w + extra[0]) / 2) & \
+                (np.abs(dz) <= (h + extra[2]) / 2)
+        for p in np.nonzero(large)[0]:
+            want.append((b, p, lx[p], ly[p], dz[p], 0.0 if inside[p] else 1.0, w, l, h))
+    got = {(int(r), int(i)): f for i, r, f in zip(idx, roi, feats)}
+    near = 0
+    for (b, p, lx, ly, dz, margin, w, l, h) in want:
+        edge = min(abs(abs(lx) - l / 2), abs(abs(ly) - w / 2), abs(abs(dz) - h / 2),
+                   abs(abs(lx) - (l + extra[1]) / 2), abs(abs(ly) - (w + extra[0]) / 2),
+                   abs(abs(dz) - (h + extra[2]) / 2))
+        if edge < 1e-4:      # a float-rounding distance from a face: either answer is right
+            near += 1
+            continue
+        f = got[(b, p)]
+        np.testing.assert_allclose(f[3:6], [lx, ly, dz], atol=2e-5)
+        np.testing.assert_allclose(f[6:12], [lx + l / 2, ly + w / 2, dz + h / 2, -lx + l / 2, -ly + w / 2,
+                                             -dz + h / 2], atol=3e-5)
+        assert f[12] == margin and np.array_equal(f[0:3], pts.numpy()[p])
+    assert len(got) >= len(want) - near and near < 20
+    # (box, point) order, and the caps keep the first hits in that order
+    order = np.lexsort((idx, roi))
+    assert np.array_equal(order, np.arange(idx.shape[0]))
+    i2, r2, f2 = orc.dynamic_point_pool(rois.numpy(), pts.numpy(), extra, 7, 50)
+    assert i2.shape[0] == 50 and np.bincount(r2).max() <= 7
+    keep = np.concatenate([np.nonzero(roi == b)[0][:7] for b in range(rois.shape[0])])[:50]
+    assert np.array_equal(i2, idx[keep]) and np.array_equal(f2, feats[keep])
+
+
+def test_grid_hash_oracle():
+    rng = np.random.default_rng(5)
+    keys = rng.choice(10 ** 7, size=3000, replace=False).astype(np.int32)
+    vals = np.arange(3000, dtype=np.int32)
+    table = orc.grid_hash_build(keys, vals)
+    assert table.shape == (4096, 2)
+    # a dictionary is the specification: every key maps to its value, others to -1
+    assert np.array_equal(orc.grid_hash_probe(keys, table), vals)
+    missing = np.setdiff1d(rng.integers(0, 10 ** 7, size=2000).astype(np.int32), keys)
+    assert (orc.grid_hash_probe(missing, table) == -1).all()
+    stored = table[table[:, 0] != -1]
+    assert stored.shape[0] == 3000 and set(map(tuple, stored)) == set(zip(keys.tolist(), vals.tolist()))
+    # probe sequence of functions.cuh:33-36: first slot key % size, step 2*key+1 (odd: full cycle)
+    k = int(keys[0])
+    first = k % 4096
+    assert table[first, 0] != -1
+    # a full table (N a power of two) still places every key
+    keys2 = rng.choice(10 ** 6, size=1024, replace=False).astype(np.int32)
+    t2 = orc.grid_hash_build(keys2, np.arange(1024, dtype=np.int32))
+    assert (t2[:, 0] != -1).all() and np.array_equal(orc.grid_hash_probe(keys2, t2), np.arange(1024))

@@ -8,6 +8,8 @@ missing.
 """
 from .scatter_op import (ScatterData, getPreSum, ingroup_inds, scatter_max, scatter_mean, scatter_sum,
                          voxelize)
+from .point_ops import GridHash, dynamic_point_pool, grid_hash_build, grid_hash_probe
 from .timer import TorchTimer
 
-__all__ = ['TorchTimer', 'scatter_sum', 'scatter_mean', 'scatter_max', 'ScatterData', 'ingroup_inds']
+__all__ = ['dynamic_point_pool', 'TorchTimer', 'ingroup_inds', 'scatter_sum', 'scatter_mean', 'scatter_max',
+           'ScatterData', 'grid_hash_build', 'grid_hash_probe', 'GridHash']

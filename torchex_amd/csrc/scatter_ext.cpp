@@ -222,6 +222,76 @@ Tensor ingroup_inds(const Tensor &seg, const OptTensor &perm, const Tensor &preS
     return out;
 }
 
+// dynamic_point_pool(rois [B,7], pts [P,3], extra_wlh, max_pts_per_box, max_all_pts)
+// -> (out_pts_idx int64 [M], out_roi_idx int64 [M], out_pts_feats float [M,13]); one host sync to read M.
+std::tuple<Tensor, Tensor, Tensor> dynamic_point_pool(const Tensor &rois, const Tensor &pts,
+                                                      std::vector<double> extra_wlh,
+                                                      int64_t max_pts_per_box, int64_t max_all_pts) {
+    check_dev(rois, "rois");
+    check_dev(pts, "pts");
+    TORCH_CHECK(rois.dim() == 2 && rois.size(1) == 7 && rois.scalar_type() == at::kFloat,
+                "rois must be float32 [num_boxes, 7]");
+    TORCH_CHECK(pts.dim() == 2 && pts.size(1) == 3 && pts.scalar_type() == at::kFloat,
+                "pts must be float32 [num_pts, 3]");
+    TORCH_CHECK(extra_wlh.size() == 3, "extra_wlh needs 3 entries");
+    TORCH_CHECK(max_all_pts >= 0 && max_pts_per_box >= 0, "caps must be non-negative");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(pts.device());
+    const int64_t B = rois.size(0), P = pts.size(0);
+    const float extra[3] = {(float)extra_wlh[0], (float)extra_wlh[1], (float)extra_wlh[2]};
+    auto iopt = pts.options().dtype(at::kInt);
+    Tensor ws = at::empty({txs_dpp_workspace_len(P, B) + 2}, iopt);
+    Tensor idx = at::empty({max_all_pts}, pts.options().dtype(at::kLong));
+    Tensor roi = at::empty({max_all_pts}, pts.options().dtype(at::kLong));
+    Tensor feats = at::empty({max_all_pts, 13}, pts.options());
+    Tensor num = at::zeros({1}, iopt);
+    check_status(txs_dynamic_point_pool(B ? rois.data_ptr<float>() : nullptr, P ? pts.data_ptr<float>() : nullptr,
+                                        B, P, extra, (int32_t)max_pts_per_box, max_all_pts, i32w(ws),
+                                        max_all_pts ? idx.data_ptr<int64_t>() : nullptr,
+                                        max_all_pts ? roi.data_ptr<int64_t>() : nullptr,
+                                        max_all_pts ? feats.data_ptr<float>() : nullptr, i32w(num),
+                                        cur_stream(pts)),
+                 "dynamic_point_pool");
+    const int64_t M = num.cpu().data_ptr<int32_t>()[0];
+    return {idx.narrow(0, 0, M), roi.narrow(0, 0, M), feats.narrow(0, 0, M)};
+}
+
+int64_t up_2n_host(int64_t n) {  // torchex/src/grid_hash/grid_hash.cpp:28-37
+    int64_t p = 1;
+    while (p < n) p <<= 1;
+    return p;
+}
+
+// build_table(coors int32 [N], values int32 [N]) -> table int32 [up_2n(N), 2]
+// (torchex/src/grid_hash/grid_hash.cpp:49-78)
+Tensor grid_hash_build(const Tensor &coors, const Tensor &values) {
+    check_i32(coors, "coors");
+    check_i32(values, "values");
+    TORCH_CHECK(coors.dim() == 1 && values.dim() == 1 && coors.numel() == values.numel(),
+                "coors and values must be 1-D of equal length");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(coors.device());
+    const int64_t N = coors.numel(), size = up_2n_host(N > 0 ? N : 1);
+    Tensor table = at::empty({size, 2}, coors.options());
+    check_status(txs_grid_hash_build(i32p(coors), i32p(values), N, table.data_ptr<int32_t>(), size, nullptr,
+                                     cur_stream(coors)),
+                 "grid_hash_build");
+    return table;
+}
+
+// probe_table(coors int32 [N], table) -> values int32 [N] (-1 where the key is absent)
+// (torchex/src/grid_hash/grid_hash.cpp:85-112)
+Tensor grid_hash_probe(const Tensor &coors, const Tensor &table) {
+    check_i32(coors, "coors");
+    check_i32(table, "table");
+    TORCH_CHECK(coors.dim() == 1, "coors must be 1-D");
+    TORCH_CHECK(table.dim() == 2 && table.size(1) == 2, "table must be [size, 2]");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(coors.device());
+    Tensor out = at::empty_like(coors);
+    check_status(txs_grid_hash_probe(i32p(coors), coors.numel(), table.data_ptr<int32_t>(), table.size(0),
+                                     i32w(out), cur_stream(coors)),
+                 "grid_hash_probe");
+    return out;
+}
+
 Tensor make_scratch(int64_t num_special, int64_t C, const Tensor &like) {
     return at::zeros({num_special * C}, like.options().dtype(at::kLong));
 }
@@ -357,6 +427,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("voxel_keys", &voxel_keys, "voxel_keys(points, range_lo, voxel_size, dims) -> (coors, keys, stats)");
     m.def("unique_plan", &unique_plan, "unique_plan(keys, key_bound, heavy_threshold, stats|None)");
     m.def("ingroup_inds", &ingroup_inds, "ingroup_inds(seg, perm|None, preSum, num_unq)");
+    m.def("dynamic_point_pool", &dynamic_point_pool, "dynamic_point_pool(rois, pts, extra_wlh, max_pts_per_box, max_all_pts)");
+    m.def("grid_hash_build", &grid_hash_build, "build_table(coors, values) -> table");
+    m.def("grid_hash_probe", &grid_hash_probe, "probe_table(coors, table) -> values");
     m.def("make_scratch", &make_scratch, "zeroed scratch table for the special voxels");
     m.def("forward", &forward, "forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, max_cnt)");
     m.def("backward", &backward, "backward(op, grad_out, arg, perm, seg, preSum, num_total)");
