@@ -152,6 +152,24 @@ def main():
     frontend["ScatterData_from_points_ms"] = wall_ms(
         lambda: T.ScatterData.from_points(pts, [0.2, 0.2, 0.2], [-75, -75, -2, 75, 75, 4]))
 
+    # the other callers of the path: points-in-boxes producer and the coordinate hash
+    gb = torch.Generator().manual_seed(11)
+    nb = 200
+    rois = torch.zeros((nb, 7))
+    rois[:, 0:2] = torch.rand((nb, 2), generator=gb) * 140 - 70
+    rois[:, 3:6] = torch.rand((nb, 3), generator=gb) * 4 + 1
+    rois[:, 6] = torch.rand((nb,), generator=gb) * 6.283
+    rois = rois.to(dev)
+    p3 = pts[:200_000, :3].contiguous()
+    frontend["dynamic_point_pool_200boxes_200kpts_ms"] = wall_ms(
+        lambda: T.dynamic_point_pool(rois, p3, [0.5, 0.5, 0.2], 512, 200_000), 10)
+    hk = torch.unique(keys).int()
+    hv = torch.arange(hk.numel(), device=dev, dtype=torch.int32)
+    table = T.grid_hash_build(hk, hv)
+    k32 = keys.int()
+    frontend["grid_hash_build_%dkeys_ms" % hk.numel()] = wall_ms(lambda: T.grid_hash_build(hk, hv), 20)
+    frontend["grid_hash_probe_1M_ms"] = wall_ms(lambda: T.grid_hash_probe(k32, table), 20)
+
     def step():
         feats.grad = None
         T.scatter_mean(feats, data).backward(g_mean)
