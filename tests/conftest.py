@@ -14,6 +14,11 @@ GOLDEN = os.path.join(ROOT, "tests", "golden")
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # a fresh checkout carries no shared objects: build the missing ones once
+    from torchex_amd import _build
+    _build.ensure_built()
+    from oracle import c_oracle
+    c_oracle.lib()
 
 
 def pytest_collection_modifyitems(config, items):

@@ -69,6 +69,16 @@ def build_all():
     build_ext()
 
 
+def ensure_built():
+    """Build what is missing (a fresh checkout has no shared objects: they are not
+    tracked).  Used by the test suite, ``bench.py`` and the smoke entry point; importing
+    ``torchex_amd`` itself never builds and raises if a piece is missing."""
+    if not os.path.exists(KERNEL_LIB):
+        build_kernels()
+    if not os.path.exists(EXT_LIB):
+        build_ext()
+
+
 if __name__ == "__main__":
     build_all()
     sys.exit(0)
