@@ -97,8 +97,8 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
 
-    from torchex_amd import _build
-    _build.ensure_built()
+    import __graft_entry__
+    __graft_entry__._load_build().ensure_built()
     import torchex_amd as T
     from torchex_amd import workloads
     from torchex_amd._native import scatter_ext

@@ -12,11 +12,21 @@ if ROOT not in sys.path:
 GOLDEN = os.path.join(ROOT, "tests", "golden")
 
 
+def _load_build():
+    """``torchex_amd/_build.py`` loaded by path: importing the package itself needs the
+    shared objects this module creates."""
+    import importlib.util
+    path = os.path.join(ROOT, "torchex_amd", "_build.py")
+    spec = importlib.util.spec_from_file_location("_torchex_amd_build", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
     # a fresh checkout carries no shared objects: build the missing ones once
-    from torchex_amd import _build
-    _build.ensure_built()
+    _load_build().ensure_built()
     from oracle import c_oracle
     c_oracle.lib()
 
