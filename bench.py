@@ -10,8 +10,10 @@ LiDAR-like sweep: N = 1,000,000 points, C = 128 fp32 features, 0.2 m voxels.
 Inputs are resident in HBM before the timed region starts.
 
 ``value`` is points per second per operator pass: ``2 * N / t_step`` (each step
-pushes the N points through two operators' forward+backward).  Per-operator
-times, GB/s and roofline fractions are in ``per_op``.
+pushes the N points through two operators' forward+backward).  Per-kernel
+durations are measured inside a second pass over the same steps, with a HIP event
+between the four entry-point calls; per-operator times, GB/s and roofline fractions
+derived from them are in ``per_kernel`` / ``per_op``.
 
 Prints ONE JSON line on stdout.
 """
@@ -35,9 +37,9 @@ HBM_PEAK_GBPS = 8000.0
 # reads half of the copied bytes on this part: factor 2.000; WRITE_SIZE: factor 1.000).
 MEASURED_TRAFFIC_BYTES = {
     "max_fwd": 525.4e6 + 334.7e6,
-    "max_bwd": 354.3e6 + 512.1e6,
+    "max_bwd": 361.9e6 + 512.1e6,
     "mean_fwd": 525.5e6 + 167.4e6,
-    "mean_bwd": 184.8e6 + 512.5e6,
+    "mean_bwd": 184.8e6 + 512.0e6,
 }
 
 
@@ -48,6 +50,8 @@ def parse():
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--kernel-iters", type=int, default=50, help="launches per per-kernel timing loop")
     p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--isolated", action="store_true",
+                   help="also time each step kernel in a back-to-back loop of its own")
     p.add_argument("--points", type=int, default=1_000_000)
     p.add_argument("--channels", type=int, default=128)
     return p.parse_args()
@@ -188,23 +192,53 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / a.steps * 1e3
 
-    # per-kernel durations: HIP events around back-to-back launches of one entry point
+    # per-kernel durations inside the step: the same four entry-point calls in the same
+    # order as the timed region above, each bracketed by HIP events recorded on the
+    # stream the kernels are launched on (so every launch sees the cache state it sees
+    # in the step, not the one a back-to-back loop of one kernel leaves behind)
     f = feats.detach()
     sc = data.scratch(C)
     plan = (data.perm, data.seg, data.preSum, data.slot_of, data.heavy_ids, sc, data.max_cnt)
+    bplan = (data.perm, data.seg, data.preSum, N)
     _, arg = scatter_ext.forward(scatter_ext.MAX, f, *plan)
+    names = ("mean_fwd", "mean_bwd", "max_fwd", "max_bwd")
+
+    def raw_step(ev=None):
+        rec = (lambda i: ev[i].record()) if ev is not None else (lambda i: None)
+        rec(0)
+        scatter_ext.forward(scatter_ext.MEAN, f, *plan)
+        rec(1)
+        scatter_ext.backward(scatter_ext.MEAN, g_mean, None, *bplan)
+        rec(2)
+        _, a2 = scatter_ext.forward(scatter_ext.MAX, f, *plan)
+        rec(3)
+        scatter_ext.backward(scatter_ext.MAX, g_max, a2, *bplan)
+        rec(4)
+
+    for _ in range(max(a.warmup, 1)):
+        raw_step()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(a.steps)]
+    torch.cuda.synchronize()
+    for e in evs:
+        raw_step(e)
+    torch.cuda.synchronize()
+    kt = {n: sum(e[i].elapsed_time(e[i + 1]) for e in evs) / len(evs) for i, n in enumerate(names)}
+    kernel_sum_ms = sum(kt.values())
+
+    # scatter_sum is not part of the step: back-to-back launches of its own kernels
     it = a.kernel_iters
-    kt = {
-        "mean_fwd": event_ms(lambda: scatter_ext.forward(scatter_ext.MEAN, f, *plan), it),
-        "mean_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MEAN, g_mean, None, data.perm, data.seg,
-                                                          data.preSum, N), it),
-        "max_fwd": event_ms(lambda: scatter_ext.forward(scatter_ext.MAX, f, *plan), it),
-        "max_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MAX, g_max, arg, data.perm, data.seg,
-                                                         data.preSum, N), it),
-        "sum_fwd": event_ms(lambda: scatter_ext.forward(scatter_ext.SUM, f, *plan), it),
-        "sum_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.SUM, g_mean, None, data.perm, data.seg,
-                                                         data.preSum, N), it),
-    }
+    kt["sum_fwd"] = event_ms(lambda: scatter_ext.forward(scatter_ext.SUM, f, *plan), it)
+    kt["sum_bwd"] = event_ms(lambda: scatter_ext.backward(scatter_ext.SUM, g_mean, None, *bplan), it)
+    isolated = None
+    if a.isolated:
+        # back-to-back launches of one entry point: upstream rows stay in the 256 MB
+        # memory-side cache between launches, so the backward kernels read faster here
+        isolated = {
+            "mean_fwd": event_ms(lambda: scatter_ext.forward(scatter_ext.MEAN, f, *plan), it),
+            "mean_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MEAN, g_mean, None, *bplan), it),
+            "max_fwd": event_ms(lambda: scatter_ext.forward(scatter_ext.MAX, f, *plan), it),
+            "max_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MAX, g_max, arg, *bplan), it),
+        }
     ab = {k: workloads.algorithmic_bytes(k, N, C, U) for k in kt}
     per_kernel = {k: {"ms": kt[k], "GBps": ab[k] / kt[k] / 1e6, "frac": ab[k] / kt[k] / 1e6 / HBM_PEAK_GBPS}
                   for k in kt}
@@ -241,11 +275,14 @@ def main():
         "roofline": roofline,
         "per_op": per_op,
         "per_kernel": per_kernel,
+        "kernel_sum_ms": kernel_sum_ms,
         "device_copy_GBps": copy_gbps,
         "index_prep_ms": prep_ms,
         "step_incl_index_prep_ms": ms_per_step + prep_ms,
         "frontend": frontend,
     }
+    if isolated is not None:
+        out["per_kernel_isolated_ms"] = isolated
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, g_mean_cpu, g_max_cpu)
     print(json.dumps(out), flush=True)
