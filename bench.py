@@ -50,10 +50,17 @@ def parse():
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--kernel-iters", type=int, default=50, help="launches per per-kernel timing loop")
     p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--no-frontend", action="store_true", help="skip the front-end timings")
     p.add_argument("--isolated", action="store_true",
                    help="also time each step kernel in a back-to-back loop of its own")
     p.add_argument("--points", type=int, default=1_000_000)
     p.add_argument("--channels", type=int, default=128)
+    p.add_argument("--workload", default="lidar_sweep",
+                   choices=("lidar_sweep", "uniform_box", "zipf_contention", "multi_sweep",
+                            "reference_test_groups"),
+                   help="lidar_sweep (default) is the workload the headline metric is quoted on; the "
+                        "others run at their own fixed sizes and ignore --points/--channels")
+    p.add_argument("--dtype", default="f32", choices=("f32", "f16", "bf16"))
     return p.parse_args()
 
 
@@ -91,43 +98,11 @@ def cpu_baseline(w, g_mean, g_max):
             "sample": f"{iters} full steps (N={w.N}, C={w.C}) of torch.scatter_reduce/index_add/gather on CPU"}
 
 
-def main():
-    a = parse()
-    if a.gpus != 1:
-        print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)",
-              file=sys.stderr)
-        sys.exit(2)
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(2)
-
-    import __graft_entry__
-    __graft_entry__._load_build().ensure_built()
-    import torchex_amd as T
-    from torchex_amd import workloads
-    from torchex_amd._native import scatter_ext
-
-    dev = torch.device("cuda:0")
-    w = workloads.lidar_sweep(N=a.points, C=a.channels, seed=2)
-    N, C, U = w.N, w.C, w.U
-    g_mean_cpu = workloads.upstream_grad(U, C, 102)
-    g_max_cpu = workloads.upstream_grad(U, C, 103)
-
-    feats = w.feats.to(dev).requires_grad_(True)
-    inv, cnts = w.unq_inv.to(dev), w.unq_cnts.to(dev)
-    g_mean, g_max = g_mean_cpu.to(dev), g_max_cpu.to(dev)
-
-    # index preparation, timed separately
-    data = T.ScatterData(inv, cnts)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(5):
-        data = T.ScatterData(inv, cnts)
-    torch.cuda.synchronize()
-    prep_ms = (time.perf_counter() - t0) / 5 * 1e3
-
-    # front-end: keys -> (unique, inverse, counts) + plan.  torch.unique followed by
-    # ScatterData sorts twice; ScatterData.from_keys sorts once.
+def frontend_timings(T, workloads, dev, N):
+    """Wall-clock timings of the callers either side of the scatter operators (voxel keys,
+    unique + plan, points-in-boxes, coordinate hash) on LiDAR-like keys."""
+    # keys -> (unique, inverse, counts) + plan.  torch.unique followed by ScatterData
+    # sorts twice; ScatterData.from_keys sorts once.
     keys_cpu, key_bound = workloads._lidar_keys(N, torch.Generator().manual_seed(2))
     keys = keys_cpu.to(dev)
 
@@ -175,6 +150,52 @@ def main():
     k32 = keys.int()
     frontend["grid_hash_build_%dkeys_ms" % hk.numel()] = wall_ms(lambda: T.grid_hash_build(hk, hv), 20)
     frontend["grid_hash_probe_1M_ms"] = wall_ms(lambda: T.grid_hash_probe(k32, table), 20)
+    return frontend
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    import __graft_entry__
+    __graft_entry__._load_build().ensure_built()
+    import torchex_amd as T
+    from torchex_amd import workloads
+    from torchex_amd._native import scatter_ext
+
+    dev = torch.device("cuda:0")
+    if a.workload == "lidar_sweep":
+        w = workloads.lidar_sweep(N=a.points, C=a.channels, seed=2)
+    else:
+        w = getattr(workloads, a.workload)()
+    N, C, U = w.N, w.C, w.U
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[a.dtype]
+    esz = 4 if a.dtype == "f32" else 2
+    g_mean_cpu = workloads.upstream_grad(U, C, 102)
+    g_max_cpu = workloads.upstream_grad(U, C, 103)
+
+    feats = w.feats.to(dev).to(tdt).requires_grad_(True)
+    inv, cnts = w.unq_inv.to(dev), w.unq_cnts.to(dev)
+    g_mean, g_max = g_mean_cpu.to(dev).to(tdt), g_max_cpu.to(dev).to(tdt)
+
+    # index preparation, timed separately
+    data = T.ScatterData(inv, cnts)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        data = T.ScatterData(inv, cnts)
+    torch.cuda.synchronize()
+    prep_ms = (time.perf_counter() - t0) / 5 * 1e3
+
+    frontend = None
+    if a.workload == "lidar_sweep" and not a.no_frontend:
+        frontend = frontend_timings(T, workloads, dev, N)
 
     def step():
         feats.grad = None
@@ -239,7 +260,7 @@ def main():
             "max_fwd": event_ms(lambda: scatter_ext.forward(scatter_ext.MAX, f, *plan), it),
             "max_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MAX, g_max, arg, *bplan), it),
         }
-    ab = {k: workloads.algorithmic_bytes(k, N, C, U) for k in kt}
+    ab = {k: workloads.algorithmic_bytes(k, N, C, U, esz) for k in kt}
     per_kernel = {k: {"ms": kt[k], "GBps": ab[k] / kt[k] / 1e6, "frac": ab[k] / kt[k] / 1e6 / HBM_PEAK_GBPS}
                   for k in kt}
     per_op = {}
@@ -252,14 +273,16 @@ def main():
     # a plain device copy of the feature matrix on the same box: the practical ceiling
     dst = torch.empty_like(f)
     copy_ms = event_ms(lambda: dst.copy_(f), 20)
-    copy_gbps = 2 * f.numel() * 4 / copy_ms / 1e6
+    copy_gbps = 2 * f.numel() * esz / copy_ms / 1e6
 
     dom = max(("max_fwd", "max_bwd", "mean_fwd", "mean_bwd"), key=lambda k: kt[k])
-    kname = {"max_fwd": "scatter_fwd_kernel<F32,4,MAX>", "mean_fwd": "scatter_fwd_kernel<F32,4,MEAN>",
-             "max_bwd": "scatter_bwd_kernel<F32,4,MAX>", "mean_bwd": "scatter_bwd_kernel<F32,4,MEAN>"}[dom]
+    row_bytes = C * esz
+    vec = next(v for v in (16, 8, 4, 2) if row_bytes % v == 0 and v >= esz) // esz   # elements per lane
+    kname = "scatter_%s_kernel<%s,%d,%s>" % (dom[-3:], a.dtype.upper(), vec, dom[:-4].upper())
     roofline = {"bound": "hbm", "kernel": kname, "achieved": per_kernel[dom]["GBps"], "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s", "frac": per_kernel[dom]["frac"],
-                "traffic": MEASURED_TRAFFIC_BYTES[dom] if (N, C) == (1_000_000, 128) else None,
+                "traffic": MEASURED_TRAFFIC_BYTES[dom]
+                if (a.workload, N, C, a.dtype) == ("lidar_sweep", 1_000_000, 128, "f32") else None,
                 "algorithmic_bytes": ab[dom], "launch_ms": kt[dom]}
 
     out = {
@@ -268,9 +291,10 @@ def main():
         "unit": "points/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "lidar_sweep N=%d C=%d fp32, voxel 0.2m, U=%d, max_cnt=%d, unsorted unq_inv"
-                               % (N, C, U, data.max_cnt),
+        "dtype": a.dtype, "data": "synthetic",
+        "config": {"workload": "%s N=%d C=%d %s, U=%d, max_cnt=%d, unsorted unq_inv%s"
+                               % (a.workload, N, C, a.dtype, U, data.max_cnt,
+                                  ", voxel 0.2m" if a.workload == "lidar_sweep" else ""),
                    "num_special_voxels": data.num_special, "heavy_threshold": data.heavy_threshold},
         "roofline": roofline,
         "per_op": per_op,
@@ -283,7 +307,7 @@ def main():
     }
     if isolated is not None:
         out["per_kernel_isolated_ms"] = isolated
-    if not a.no_cpu_baseline:
+    if not a.no_cpu_baseline and a.dtype == "f32":
         out["cpu_baseline"] = cpu_baseline(w, g_mean_cpu, g_max_cpu)
     print(json.dumps(out), flush=True)
 

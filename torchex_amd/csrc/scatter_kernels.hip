@@ -963,11 +963,13 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
         // than a chunk, so a chunk touches at most one at each end)
     };
 
-    // Fold one loaded row (position l, voxel sg) into the running reduction.
-    // `valid` only gates state changes: the loaded registers are consumed on a
-    // straight-line path so the compiler can count outstanding loads exactly.
-    auto add_row = [&](const Pack<raw, VEC> &v, int sg, int row, int l, bool valid) {
-        if (valid && sg != cur) {
+    // Fold one loaded row (position l, voxel sg) into the running reduction.  With
+    // kGate the row counts only when `valid` (a slot past the range in the last
+    // batch of a chunk); the loaded registers are consumed on a straight-line path
+    // either way so the compiler can count outstanding loads exactly.
+    auto add_row = [&](auto gate, const Pack<raw, VEC> &v, int sg, int row, int l, bool valid) {
+        constexpr bool kGate = decltype(gate)::value;
+        if ((!kGate || valid) && sg != cur) {
             flush(l);
             cur = sg;
             run_l0 = l;
@@ -987,13 +989,23 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                 // mode also takes an equal value whose key is smaller.
                 bool take = x > acc[k];
                 if (kRef) take |= (x == acc[k]) && ((unsigned)tag < (unsigned)idx[k]);
-                take &= valid;
+                if (kGate) take &= valid;
                 acc[k] = take ? x : acc[k];
                 idx[k] = take ? tag : idx[k];
             } else {
-                acc[k] += valid ? x : 0.0f;
+                acc[k] += (!kGate || valid) ? x : 0.0f;
             }
         }
+    };
+
+    // Row r of the feature matrix at this lane's columns: one 64-bit multiply-add.
+    // A row index outside the matrix (only a corrupt plan has one) is clamped.
+    const char *lane_base = reinterpret_cast<const char *>(feats) + (size_t)col * sizeof(raw);
+    const unsigned row_bytes = (unsigned)C * (unsigned)sizeof(raw);
+    const unsigned last_row = (unsigned)(N - 1);
+    auto row_ptr = [&](int r) -> const raw * {
+        const unsigned rc = min((unsigned)r, last_row);
+        return reinterpret_cast<const raw *>(lane_base + (unsigned long long)rc * row_bytes);
     };
 
     // Every slot of a batch issues a load (slots past the range re-load the
@@ -1005,18 +1017,23 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     auto issue = [&](Batch &bt, int l) {
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
-            const int ll = l + i;
-            const int lc = min(ll, lb_fast - 1);
-            const int r = perm_s[lc - 1];
-            const bool valid = ll < lb_fast && (unsigned)r < (unsigned)N;
+            const int lc = min(l + i, lb_fast - 1);
             bt.segs[i] = seg_s[lc];
-            bt.rows[i] = valid ? r : -1;
-            bt.v[i] = ld_stream<raw, VEC>(feats + (size_t)((unsigned)r < (unsigned)N ? r : 0) * C + col);
+            bt.rows[i] = perm_s[lc - 1];
+            bt.v[i] = ld_stream<raw, VEC>(row_ptr(bt.rows[i]));
         }
     };
-    auto consume = [&](const Batch &bt, int l) {
+    // A batch that lies wholly inside the range needs no per-row gate; only the
+    // last batch of a chunk can hold slots past the range.
+    auto consume_full = [&](const Batch &bt, int l) {
 #pragma unroll
-        for (int i = 0; i < kBatch; ++i) add_row(bt.v[i], bt.segs[i], bt.rows[i], l + i, bt.rows[i] >= 0);
+        for (int i = 0; i < kBatch; ++i)
+            add_row(std::false_type{}, bt.v[i], bt.segs[i], bt.rows[i], l + i, true);
+    };
+    auto consume_last = [&](const Batch &bt, int l) {
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i)
+            add_row(std::true_type{}, bt.v[i], bt.segs[i], bt.rows[i], l + i, l + i < lb_fast);
     };
 
     // Positions staged in LDS go through the double-buffered loop; the rare rest
@@ -1030,25 +1047,25 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     for (int l = la;;) {
         int ln = l + kBatch;
         if (ln >= lb_fast) {
-            consume(b0, l);
+            consume_last(b0, l);
             break;
         }
         issue(b1, ln);
-        consume(b0, l);
+        consume_full(b0, l);
         l = ln;
         ln = l + kBatch;
         if (ln >= lb_fast) {
-            consume(b1, l);
+            consume_last(b1, l);
             break;
         }
         issue(b0, ln);
-        consume(b1, l);
+        consume_full(b1, l);
         l = ln;
     }
     for (int l = lb_fast; l < lb; ++l) {
         const int r = row_at(l);
         if ((unsigned)r >= (unsigned)N) continue;
-        add_row(ld_stream<raw, VEC>(feats + (size_t)r * C + col), seg_at(l), r, l, true);
+        add_row(std::false_type{}, ld_stream<raw, VEC>(row_ptr(r)), seg_at(l), r, l, true);
     }
     flush(lb);
     };  // reduce_chunk
