@@ -1,7 +1,8 @@
 """In-tree build of the two native pieces (run on a CPU-only machine; hipcc
 cross-compiles for gfx950):
 
-``libtorchex_scatter.so``  HIP kernels + C ABI, built with hipcc, no torch in it.
+``libtorchex_scatter.so``  HIP kernels + C ABI (three translation units under
+                           ``csrc/``), built with hipcc, no torch in it.
 ``scatter_ext*.so``        the PyTorch C++ extension module, built with the host
                            compiler against the torch headers; links to the
                            library above through ``$ORIGIN``.
@@ -24,9 +25,11 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 # packed-fp32 code generation is switched off for every HIP translation unit
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+KERNEL_SOURCES = ["plan_kernels.hip", "frontend_kernels.hip", "scatter_kernels.hip"]
+OBJ_DIR = os.path.join(PKG, "_obj")
 
 
 def _run(cmd):
@@ -35,9 +38,19 @@ def _run(cmd):
 
 
 def build_kernels():
+    """Compile the HIP translation units side by side, then link them into one library."""
     hipcc = os.path.join(ROCM, "bin", "hipcc")
-    src = os.path.join(CSRC, "scatter_kernels.hip")
-    _run([hipcc, *HIPCC_FLAGS, "-I" + INCLUDE, "-o", KERNEL_LIB, src])
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    jobs = []
+    for name in KERNEL_SOURCES:
+        obj = os.path.join(OBJ_DIR, os.path.splitext(name)[0] + ".o")
+        cmd = [hipcc, *HIPCC_FLAGS, "-I" + INCLUDE, "-c", os.path.join(CSRC, name), "-o", obj]
+        print("+", " ".join(cmd), flush=True)
+        jobs.append((cmd, obj, subprocess.Popen(cmd)))
+    for cmd, _, proc in jobs:
+        if proc.wait() != 0:
+            raise subprocess.CalledProcessError(proc.returncode, cmd)
+    _run([hipcc, "--offload-arch=gfx950", "-fPIC", "-shared", "-o", KERNEL_LIB, *[obj for _, obj, _ in jobs]])
     return KERNEL_LIB
 
 

@@ -1,0 +1,426 @@
+// The callers on either side of the scatter operators: voxel keys from points,
+// the unique / inverse / counts triple (from the same sort the scatter plan uses),
+// the rank of an element inside its group, points-in-boxes pooling, and the
+// coordinate hash table.
+//
+// Reference behaviour being replaced: voxelize_single
+// (test/test_incremental_mask.py:20-26), ingroup_inds
+// (torchex/src/ingroup_inds/ingroup_inds_kernel.cu:17-30), dynamic_point_pool
+// (torchex/src/dynamic_point_pool/dynamic_point_pool_kernel.cu:22-170,280-310),
+// grid_hash (torchex/src/grid_hash/grid_hash_kernel.cu:19-49,
+// torchex/src/utils/functions.cuh:30-64).
+
+#include "txs_common.h"
+
+namespace {
+
+using txs_detail::exclusive_scan;
+using txs_detail::scan_tiles;
+
+__global__ void fill_i32_kernel(int *p, long n, int value) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = value;
+}
+
+// ------------------------------------------------ voxelization front-end --
+
+// torch.div(a, b, rounding_mode='floor') for fp32 (c10::div_floor_floating,
+// c10/util/generic_math.h): Python's floor division, not floor(a / b).
+__device__ __forceinline__ float div_floor_f32(float a, float b) {
+    if (b == 0.0f) return a / b;
+    const float mod = fmodf(a, b);
+    float div = (a - mod) / b;
+    if ((mod != 0.0f) && ((b < 0.0f) != (mod < 0.0f))) div -= 1.0f;
+    float fl;
+    if (div != 0.0f) {
+        fl = floorf(div);
+        if (div - fl > 0.5f) fl += 1.0f;
+    } else {
+        fl = copysignf(0.0f, a / b);
+    }
+    return fl;
+}
+
+// coors = floor((p - lo) / voxel) per axis, key = (x * Y + y) * Z + z
+// (test/test_incremental_mask.py:20-26, operator_py/incremental_points.py:18-19)
+__global__ void voxel_keys_kernel(const float *__restrict__ pts, long n, int stride, float lo0,
+                                  float lo1, float lo2, float v0, float v1, float v2, int d0, int d1,
+                                  int d2, int *__restrict__ coors, int *__restrict__ keys,
+                                  int *__restrict__ stats) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float *p = pts + i * stride;
+    const int x = (int)div_floor_f32(p[0] - lo0, v0);
+    const int y = (int)div_floor_f32(p[1] - lo1, v1);
+    const int z = (int)div_floor_f32(p[2] - lo2, v2);
+    if (coors) {
+        coors[i * 3 + 0] = x;
+        coors[i * 3 + 1] = y;
+        coors[i * 3 + 2] = z;
+    }
+    const bool ok = (unsigned)x < (unsigned)d0 && (unsigned)y < (unsigned)d1 && (unsigned)z < (unsigned)d2;
+    if (!ok) stats[TXS_STAT_OUT_OF_RANGE] = 1;
+    keys[i] = ok ? (x * d1 + y) * d2 + z : 0;
+}
+
+// 1 where a new run of equal keys starts
+__global__ void run_flags_kernel(const int *__restrict__ ks, long n, int *__restrict__ flags) {
+    long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j < n) flags[j] = (j == 0 || ks[j] != ks[j - 1]) ? 1 : 0;
+}
+
+// What torch.unique(keys, return_inverse=True, return_counts=True) returns,
+// from the sorted keys and the exclusive scan `ex` of the run-start flags,
+// plus the plan arrays: run index rid = ex[j] + flag - 1.
+__global__ void unique_finish_kernel(const int *__restrict__ ks, const int *__restrict__ perm,
+                                     const int *__restrict__ ex, long n, int *__restrict__ seg,
+                                     int *__restrict__ inv, int *__restrict__ unq,
+                                     int *__restrict__ preSum, int *__restrict__ stats) {
+    long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    const bool flag = (j == 0 || ks[j] != ks[j - 1]);
+    const int rid = ex[j] + (flag ? 1 : 0) - 1;
+    const int row = stats[TXS_STAT_UNSORTED] ? perm[j] : (int)j;
+    seg[j] = rid;
+    if ((unsigned)row < (unsigned)n) inv[row] = rid;
+    if (flag) {
+        unq[rid] = ks[j];
+        preSum[rid] = (int)j;
+    }
+    if (j == n - 1) {
+        preSum[rid + 1] = (int)n;
+        stats[TXS_STAT_NUM_UNQ] = rid + 1;
+    }
+}
+
+// rank of every element inside its group (operator_py/ingroup_inds_op.py,
+// src/ingroup_inds/ingroup_inds_kernel.cu:17-30): sorted position minus the
+// group's first position; ascending with the element's index, where the
+// reference's atomic counter hands ranks out in arbitrary order.
+__global__ void ingroup_inds_kernel(const int *__restrict__ seg, const int *__restrict__ perm,
+                                    const int *__restrict__ preSum, long n, int U,
+                                    long long *__restrict__ out) {
+    long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    const int u = seg[j] & kIdMask;
+    const int row = perm ? perm[j] : (int)j;
+    if ((unsigned)u < (unsigned)U && (unsigned)row < (unsigned)n) out[row] = (long long)(j - preSum[u]);
+}
+
+// ------------------------------------------------------ dynamic point pool --
+// Points inside (enlarged) rotated boxes, with 13 box-relative numbers per hit
+// (torchex/src/dynamic_point_pool/dynamic_point_pool_kernel.cu:22-170,280-310).
+// The reference compacts the hits with two atomic counters, so their order and,
+// when a cap is hit, the surviving subset depend on thread timing.  Here the
+// hits are counted per (box, tile of 256 points), scanned, and written in
+// (box, point) order: the outcome the reference's own comment calls the usual
+// one ("out_roi_idx is automatically sorted"), made deterministic.
+
+constexpr int kDppInfo = 13;
+
+struct DppBox {
+    float cx, cy, czc, w, l, h, cosa, sina, large_w, large_l, large_h, cz_bottom;
+};
+
+// per-box constants, computed once so both passes see identical numbers; the
+// rotation terms are evaluated in double and rounded (within an ulp of any cosf)
+__global__ void dpp_box_kernel(const float *__restrict__ rois, int B, float extra_w, float extra_l,
+                               float extra_h, DppBox *__restrict__ boxes) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= B) return;
+    const float *r = rois + (size_t)b * 7;
+    DppBox bx;
+    bx.cx = r[0];
+    bx.cy = r[1];
+    bx.cz_bottom = r[2];
+    bx.w = r[3];
+    bx.l = r[4];
+    bx.h = r[5];
+    bx.large_w = bx.w + extra_w;
+    bx.large_l = bx.l + extra_l;
+    bx.large_h = bx.h + extra_h;
+    bx.czc = (float)((double)r[2] + (double)bx.h / 2.0);  // bottom centre -> centre (:46)
+    const float rot = (float)((double)r[6] + 3.14159265358979323846 / 2);  // (:24)
+    bx.cosa = (float)cos((double)rot);
+    bx.sina = (float)sin((double)rot);
+    boxes[b] = bx;
+}
+
+// 0: outside the enlarged box, 1: in the margin, 2: inside the box (:33-71)
+__device__ __forceinline__ int dpp_test(const DppBox &bx, float x, float y, float z, float &local_x,
+                                        float &local_y) {
+#pragma clang fp contract(off)
+    if ((double)fabsf(z - bx.czc) > (double)bx.large_h / 2.0) return 0;
+    const float sx = x - bx.cx, sy = y - bx.cy;
+    local_x = sx * bx.cosa + sy * (-bx.sina);
+    local_y = sx * bx.sina + sy * bx.cosa;
+    const double lx = local_x, ly = local_y;
+    const bool in_box = (lx > -(double)bx.l / 2.0) & (lx < (double)bx.l / 2.0) &
+                        (ly > -(double)bx.w / 2.0) & (ly < (double)bx.w / 2.0) &
+                        ((double)fabsf(z - bx.czc) < (double)bx.h / 2.0);
+    const bool in_large = (lx > -(double)bx.large_l / 2.0) & (lx < (double)bx.large_l / 2.0) &
+                          (ly > -(double)bx.large_w / 2.0) & (ly < (double)bx.large_w / 2.0);
+    return in_box ? 2 : (in_large ? 1 : 0);
+}
+
+// hits per (box, tile); grid (tiles, boxes)
+__global__ __launch_bounds__(kThreads) void dpp_count_kernel(const float *__restrict__ pts, int P,
+                                                             const DppBox *__restrict__ boxes,
+                                                             int n_tiles, int *__restrict__ counts) {
+    __shared__ int wsum[kThreads / 64];
+    const int p = blockIdx.x * kThreads + threadIdx.x;
+    const DppBox bx = boxes[blockIdx.y];
+    bool hit = false;
+    if (p < P) {
+        float lx, ly;
+        hit = dpp_test(bx, pts[(size_t)p * 3], pts[(size_t)p * 3 + 1], pts[(size_t)p * 3 + 2], lx, ly) > 0;
+    }
+    const int c = __popcll(__ballot(hit));
+    if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int t = 0;
+        for (int k = 0; k < kThreads / 64; ++k) t += wsum[k];
+        counts[(size_t)blockIdx.y * n_tiles + blockIdx.x] = t;
+    }
+}
+
+// per-box kept count = min(hits, cap), exclusive scan over boxes, total (one workgroup)
+__global__ __launch_bounds__(kThreads) void dpp_box_base_kernel(const int *__restrict__ scanned,
+                                                                int B, int n_tiles, int cap,
+                                                                int max_all, int *__restrict__ box_base,
+                                                                int *__restrict__ total_out) {
+    int carry = 0;
+    for (int base = 0; base < B; base += kThreads) {
+        const int b = base + threadIdx.x;
+        int kept = 0;
+        if (b < B) kept = min(scanned[(size_t)(b + 1) * n_tiles] - scanned[(size_t)b * n_tiles], cap);
+        int tot;
+        const int ex = block_exclusive_scan(kept, &tot);
+        if (b < B) box_base[b] = carry + ex;
+        carry += tot;
+    }
+    if (threadIdx.x == 0) total_out[0] = min(carry, max_all);
+}
+
+// second pass: same test, rank of the hit inside its box, compact write
+__global__ __launch_bounds__(kThreads) void dpp_write_kernel(
+    const float *__restrict__ pts, int P, const DppBox *__restrict__ boxes, int n_tiles,
+    const int *__restrict__ scanned, const int *__restrict__ box_base, int cap, int max_all,
+    long long *__restrict__ out_pts_idx, long long *__restrict__ out_roi_idx,
+    float *__restrict__ out_feats) {
+#pragma clang fp contract(off)
+    __shared__ int wsum[kThreads / 64];
+    const int b = blockIdx.y;
+    const int p = blockIdx.x * kThreads + threadIdx.x;
+    const DppBox bx = boxes[b];
+    int flag = 0;
+    float x = 0.f, y = 0.f, z = 0.f, lx = 0.f, ly = 0.f;
+    if (p < P) {
+        x = pts[(size_t)p * 3];
+        y = pts[(size_t)p * 3 + 1];
+        z = pts[(size_t)p * 3 + 2];
+        flag = dpp_test(bx, x, y, z, lx, ly);
+    }
+    const unsigned long long m = __ballot(flag > 0);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (lane == 0) wsum[w] = __popcll(m);
+    __syncthreads();
+    if (flag == 0) return;
+    int rank = __popcll(m & ((1ull << lane) - 1ull));
+    for (int k = 0; k < w; ++k) rank += wsum[k];
+    rank += scanned[(size_t)b * n_tiles + blockIdx.x] - scanned[(size_t)b * n_tiles];
+    if (rank >= cap) return;
+    const long pos = (long)box_base[b] + rank;
+    if (pos >= max_all) return;
+    const float local_z = (float)((double)z - ((double)bx.cz_bottom + (double)bx.h / 2.0));  // (:103)
+    float *f = out_feats + pos * kDppInfo;
+    out_pts_idx[pos] = p;
+    out_roi_idx[pos] = b;
+    f[0] = x;
+    f[1] = y;
+    f[2] = z;
+    f[3] = lx;
+    f[4] = ly;
+    f[5] = local_z;
+    f[6] = lx + bx.l / 2;
+    f[7] = ly + bx.w / 2;
+    f[8] = local_z + bx.h / 2;
+    f[9] = -lx + bx.l / 2;
+    f[10] = -ly + bx.w / 2;
+    f[11] = -local_z + bx.h / 2;
+    f[12] = flag == 1 ? 1.0f : 0.0f;
+}
+
+// ------------------------------------------------------------- grid hash --
+// Open-addressing table of (key, value) int32 pairs with the reference's probe
+// sequence (torchex/src/utils/functions.cuh:30-64, double hashing with an odd
+// step over a power-of-two table).  A slot is one 64-bit word (key in the low
+// half, value in the high half, as the reference's [size, 2] int32 tensor lays
+// them out) claimed with a single 64-bit compare-and-swap, so key and value
+// appear together.
+
+__device__ __forceinline__ int grid_hash_slot(long long key, int probe_i, int table_size) {
+    return (int)((key % table_size + probe_i * (key * 2 + 1)) % table_size);
+}
+
+__global__ void grid_hash_build_kernel(const int *__restrict__ keys, const int *__restrict__ values,
+                                       unsigned long long *__restrict__ table, int table_size, long n,
+                                       int *__restrict__ fail) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int key = keys[i];
+    const unsigned long long word =
+        ((unsigned long long)(unsigned)values[i] << 32) | (unsigned long long)(unsigned)key;
+    const unsigned long long empty = ~0ull;  // (-1, -1)
+    for (int t = 0; t < table_size; ++t) {
+        const int s = grid_hash_slot(key, t, table_size);
+        if ((unsigned)s >= (unsigned)table_size) break;  // negative key
+        if (atomicCAS(table + s, empty, word) == empty) return;
+    }
+    if (fail) fail[0] = 1;  // table full or key negative (the reference asserts)
+}
+
+__global__ void grid_hash_probe_kernel(const int *__restrict__ keys,
+                                       const unsigned long long *__restrict__ table, int table_size,
+                                       long n, int *__restrict__ out) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int key = keys[i];
+    int v = -1;
+    for (int t = 0; t < table_size; ++t) {
+        const int s = grid_hash_slot(key, t, table_size);
+        if ((unsigned)s >= (unsigned)table_size) break;
+        const unsigned long long word = table[s];
+        const int slot_key = (int)(unsigned)(word & 0xffffffffull);
+        if (slot_key == key) {
+            v = (int)(unsigned)(word >> 32);
+            break;
+        }
+        // An empty slot on the probe sequence proves the key was never inserted
+        // (no deletions).  The reference keeps scanning all table_size slots
+        // before giving up (functions.cuh:54-63), with the same answer.
+        if (slot_key == -1) break;
+    }
+    out[i] = v;
+}
+
+}  // namespace
+
+extern "C" {
+
+int txs_voxel_keys(const float *points, int64_t num_total, int64_t point_stride,
+                   const float *range_lo, const float *voxel_size, const int32_t *dims,
+                   int32_t *coors, int32_t *keys, int32_t *stats, void *stream) {
+    if (!fits_i32(num_total) || point_stride < 3 || !range_lo || !voxel_size || !dims || !stats)
+        return TXS_ERR_INVALID_ARG;
+    const long long cells = (long long)dims[0] * dims[1] * dims[2];
+    if (dims[0] <= 0 || dims[1] <= 0 || dims[2] <= 0 || !fits_i32(cells)) return TXS_ERR_INVALID_ARG;
+    if (num_total == 0) return TXS_OK;
+    if (!points || !keys) return TXS_ERR_INVALID_ARG;
+    voxel_keys_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+        points, num_total, (int)point_stride, range_lo[0], range_lo[1], range_lo[2], voxel_size[0],
+        voxel_size[1], voxel_size[2], dims[0], dims[1], dims[2], coors, keys, stats);
+    return status_of(hipGetLastError());
+}
+
+int64_t txs_unique_workspace_len(int64_t num_total) { return num_total + scan_tiles(num_total + 1) + 17; }
+
+int txs_unique_runs(const int32_t *sorted_keys, const int32_t *perm, int64_t num_total,
+                    int32_t *unique_ws, int32_t *seg, int32_t *unq_inv, int32_t *unq_keys,
+                    int32_t *preSum, int32_t *stats, void *stream) {
+    if (!fits_i32(num_total) || !stats || !preSum) return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    if (num_total == 0) {
+        fill_i32_kernel<<<dim3(1), dim3(64), 0, st>>>(preSum, 1, 0);
+        return status_of(hipGetLastError());
+    }
+    if (!sorted_keys || !perm || !unique_ws || !seg || !unq_inv || !unq_keys) return TXS_ERR_INVALID_ARG;
+    const long n = num_total;
+    int *flags = unique_ws;
+    int *scan_ws = unique_ws + n;
+    run_flags_kernel<<<dim3(blocks_for(n)), dim3(kThreads), 0, st>>>(sorted_keys, n, flags);
+    if (exclusive_scan(flags, n, flags, n, scan_ws, st) != hipSuccess) return TXS_ERR_LAUNCH;
+    unique_finish_kernel<<<dim3(blocks_for(n)), dim3(kThreads), 0, st>>>(sorted_keys, perm, flags, n, seg,
+                                                                       unq_inv, unq_keys, preSum, stats);
+    return status_of(hipGetLastError());
+}
+
+int txs_ingroup_inds(const int32_t *seg, const int32_t *perm, const int32_t *preSum,
+                     int64_t num_total, int64_t num_unq, int64_t *out, void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_unq)) return TXS_ERR_INVALID_ARG;
+    if (num_total == 0) return TXS_OK;
+    if (!seg || !preSum || !out || num_unq <= 0) return TXS_ERR_INVALID_ARG;
+    ingroup_inds_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+        seg, perm, preSum, num_total, (int)num_unq, (long long *)out);
+    return status_of(hipGetLastError());
+}
+
+int64_t txs_dpp_workspace_len(int64_t num_pts, int64_t num_boxes) {
+    const int64_t tiles = (num_pts + kThreads - 1) / kThreads;
+    const int64_t cells = num_boxes * tiles + 1;
+    // box constants, (box, tile) counts, scan workspace, box bases
+    return (int64_t)(sizeof(DppBox) / sizeof(int)) * num_boxes + cells + scan_tiles(cells + 1) + 1 +
+           num_boxes + 16;
+}
+
+int txs_dynamic_point_pool(const float *rois, const float *pts, int64_t num_boxes, int64_t num_pts,
+                           const float *extra_wlh, int32_t max_pts_per_box, int64_t max_all_pts,
+                           int32_t *workspace, int64_t *out_pts_idx, int64_t *out_roi_idx,
+                           float *out_pts_feats, int32_t *num_out, void *stream) {
+    if (!fits_i32(num_boxes) || !fits_i32(num_pts) || !fits_i32(max_all_pts) || max_pts_per_box < 0 ||
+        !extra_wlh || !num_out)
+        return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    if (num_boxes == 0 || num_pts == 0) {
+        fill_i32_kernel<<<dim3(1), dim3(64), 0, st>>>(num_out, 1, 0);
+        return status_of(hipGetLastError());
+    }
+    if (!rois || !pts || !workspace || !out_pts_idx || !out_roi_idx || !out_pts_feats)
+        return TXS_ERR_INVALID_ARG;
+    const int B = (int)num_boxes, P = (int)num_pts;
+    const int n_tiles = (P + kThreads - 1) / kThreads;
+    const long cells = (long)B * n_tiles;
+    if (!fits_i32(cells + 1) || B > 65535) return TXS_ERR_INVALID_ARG;
+    DppBox *boxes = reinterpret_cast<DppBox *>(workspace);
+    int *counts = workspace + (sizeof(DppBox) / sizeof(int)) * (size_t)B;
+    int *scan_ws = counts + cells + 1;
+    int *box_base = scan_ws + scan_tiles(cells + 2) + 1;
+    dpp_box_kernel<<<dim3(blocks_for(B)), dim3(kThreads), 0, st>>>(rois, B, extra_wlh[0], extra_wlh[1],
+                                                                 extra_wlh[2], boxes);
+    dpp_count_kernel<<<dim3(n_tiles, B), dim3(kThreads), 0, st>>>(pts, P, boxes, n_tiles, counts);
+    if (exclusive_scan(counts, cells, counts, cells + 1, scan_ws, st) != hipSuccess) return TXS_ERR_LAUNCH;
+    dpp_box_base_kernel<<<dim3(1), dim3(kThreads), 0, st>>>(counts, B, n_tiles, max_pts_per_box,
+                                                           (int)max_all_pts, box_base, num_out);
+    dpp_write_kernel<<<dim3(n_tiles, B), dim3(kThreads), 0, st>>>(
+        pts, P, boxes, n_tiles, counts, box_base, max_pts_per_box, (int)max_all_pts,
+        (long long *)out_pts_idx, (long long *)out_roi_idx, out_pts_feats);
+    return status_of(hipGetLastError());
+}
+
+int txs_grid_hash_build(const int32_t *keys, const int32_t *values, int64_t num_keys, int32_t *table,
+                        int64_t table_size, int32_t *fail_flag, void *stream) {
+    if (!fits_i32(num_keys) || !fits_i32(table_size) || table_size <= 0 || !table) return TXS_ERR_INVALID_ARG;
+    if ((table_size & (table_size - 1)) != 0 || ((uintptr_t)table & 7) != 0) return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    fill_i32_kernel<<<dim3(blocks_for(2 * table_size)), dim3(kThreads), 0, st>>>(table, 2 * table_size, -1);
+    if (num_keys > 0) {
+        if (!keys || !values || num_keys > table_size) return TXS_ERR_INVALID_ARG;
+        grid_hash_build_kernel<<<dim3(blocks_for(num_keys)), dim3(kThreads), 0, st>>>(
+            keys, values, (unsigned long long *)table, (int)table_size, num_keys, fail_flag);
+    }
+    return status_of(hipGetLastError());
+}
+
+int txs_grid_hash_probe(const int32_t *keys, int64_t num_keys, const int32_t *table,
+                        int64_t table_size, int32_t *out_values, void *stream) {
+    if (!fits_i32(num_keys) || !fits_i32(table_size) || table_size <= 0 || !table) return TXS_ERR_INVALID_ARG;
+    if ((table_size & (table_size - 1)) != 0 || ((uintptr_t)table & 7) != 0) return TXS_ERR_INVALID_ARG;
+    if (num_keys == 0) return TXS_OK;
+    if (!keys || !out_values) return TXS_ERR_INVALID_ARG;
+    grid_hash_probe_kernel<<<dim3(blocks_for(num_keys)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+        keys, (const unsigned long long *)table, (int)table_size, num_keys, out_values);
+    return status_of(hipGetLastError());
+}
+
+}  // extern "C"
