@@ -51,6 +51,10 @@ def parse():
     p.add_argument("--kernel-iters", type=int, default=50, help="launches per per-kernel timing loop")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-frontend", action="store_true", help="skip the front-end timings")
+    p.add_argument("--sorted-input", action="store_true",
+                   help="also time the step on the same points delivered grouped by voxel "
+                        "(off by default so that a profile of the default command holds one "
+                        "population of launches per kernel)")
     p.add_argument("--isolated", action="store_true",
                    help="also time each step kernel in a back-to-back loop of its own")
     p.add_argument("--points", type=int, default=1_000_000)
@@ -89,13 +93,40 @@ def cpu_baseline(w, g_mean, g_max):
     torch.set_num_threads(threads)
     tor.step_mean_max(w.feats, w.unq_inv, w.unq_cnts, g_mean, g_max)   # warm-up
     iters, t0 = 0, time.perf_counter()
-    while iters < 3 or (time.perf_counter() - t0 < 10.0 and iters < 10):
+    while iters < 3 or (time.perf_counter() - t0 < 12.0 and iters < 40):
         tor.step_mean_max(w.feats, w.unq_inv, w.unq_cnts, g_mean, g_max)
         iters += 1
     dt = (time.perf_counter() - t0) / iters
     return {"value": 2 * w.N / dt, "unit": "points/s", "cores": torch.get_num_threads(),
             "kind": "port", "ms_per_step": dt * 1e3,
             "sample": f"{iters} full steps (N={w.N}, C={w.C}) of torch.scatter_reduce/index_add/gather on CPU"}
+
+
+def instrumented_steps(scatter_ext, f, g_mean, g_max, plan, bplan, steps, warmup):
+    """Average duration (ms) of each of the step's four entry-point calls, issued in step
+    order with a HIP event between them."""
+    names = ("mean_fwd", "mean_bwd", "max_fwd", "max_bwd")
+
+    def raw_step(ev=None):
+        rec = (lambda i: ev[i].record()) if ev is not None else (lambda i: None)
+        rec(0)
+        scatter_ext.forward(scatter_ext.MEAN, f, *plan)
+        rec(1)
+        scatter_ext.backward(scatter_ext.MEAN, g_mean, None, *bplan)
+        rec(2)
+        _, a2 = scatter_ext.forward(scatter_ext.MAX, f, *plan)
+        rec(3)
+        scatter_ext.backward(scatter_ext.MAX, g_max, a2, *bplan)
+        rec(4)
+
+    for _ in range(max(warmup, 1)):
+        raw_step()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    for e in evs:
+        raw_step(e)
+    torch.cuda.synchronize()
+    return {n: sum(e[i].elapsed_time(e[i + 1]) for e in evs) / len(evs) for i, n in enumerate(names)}
 
 
 def frontend_timings(T, workloads, dev, N):
@@ -222,29 +253,23 @@ def main():
     plan = (data.perm, data.seg, data.preSum, data.slot_of, data.heavy_ids, sc, data.max_cnt)
     bplan = (data.perm, data.seg, data.preSum, N)
     _, arg = scatter_ext.forward(scatter_ext.MAX, f, *plan)
-    names = ("mean_fwd", "mean_bwd", "max_fwd", "max_bwd")
-
-    def raw_step(ev=None):
-        rec = (lambda i: ev[i].record()) if ev is not None else (lambda i: None)
-        rec(0)
-        scatter_ext.forward(scatter_ext.MEAN, f, *plan)
-        rec(1)
-        scatter_ext.backward(scatter_ext.MEAN, g_mean, None, *bplan)
-        rec(2)
-        _, a2 = scatter_ext.forward(scatter_ext.MAX, f, *plan)
-        rec(3)
-        scatter_ext.backward(scatter_ext.MAX, g_max, a2, *bplan)
-        rec(4)
-
-    for _ in range(max(a.warmup, 1)):
-        raw_step()
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(a.steps)]
-    torch.cuda.synchronize()
-    for e in evs:
-        raw_step(e)
-    torch.cuda.synchronize()
-    kt = {n: sum(e[i].elapsed_time(e[i + 1]) for e in evs) / len(evs) for i, n in enumerate(names)}
+    kt = instrumented_steps(scatter_ext, f, g_mean, g_max, plan, bplan, a.steps, a.warmup)
     kernel_sum_ms = sum(kt.values())
+
+    # the same points delivered grouped by voxel, which is the only order the reference's
+    # kernels accept (its getPreSum needs sorted ids): no row permutation, sequential writes
+    sorted_input = None
+    if a.sorted_input and not data.is_sorted:
+        order = torch.sort(inv, stable=True)[1]
+        f_s = f[order].contiguous()
+        data_s = T.ScatterData(inv[order].contiguous(), cnts)
+        plan_s = (data_s.perm, data_s.seg, data_s.preSum, data_s.slot_of, data_s.heavy_ids,
+                  data_s.scratch(C), data_s.max_cnt)
+        kts = instrumented_steps(scatter_ext, f_s, g_mean, g_max, plan_s,
+                                 (data_s.perm, data_s.seg, data_s.preSum, N), a.steps, a.warmup)
+        sorted_input = {"per_kernel_ms": kts, "kernel_sum_ms": sum(kts.values()),
+                        "points_per_s": 2 * N / sum(kts.values()) * 1e3}
+        del f_s, data_s, plan_s, order
 
     # scatter_sum is not part of the step: back-to-back launches of its own kernels
     it = a.kernel_iters
@@ -292,14 +317,16 @@ def main():
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": a.dtype, "data": "synthetic",
-        "config": {"workload": "%s N=%d C=%d %s, U=%d, max_cnt=%d, unsorted unq_inv%s"
+        "config": {"workload": "%s N=%d C=%d %s, U=%d, max_cnt=%d, %s unq_inv%s"
                                % (a.workload, N, C, a.dtype, U, data.max_cnt,
+                                  "sorted" if data.is_sorted else "unsorted",
                                   ", voxel 0.2m" if a.workload == "lidar_sweep" else ""),
                    "num_special_voxels": data.num_special, "heavy_threshold": data.heavy_threshold},
         "roofline": roofline,
         "per_op": per_op,
         "per_kernel": per_kernel,
         "kernel_sum_ms": kernel_sum_ms,
+        "sorted_input": sorted_input,
         "device_copy_GBps": copy_gbps,
         "index_prep_ms": prep_ms,
         "step_incl_index_prep_ms": ms_per_step + prep_ms,
