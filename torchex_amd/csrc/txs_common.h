@@ -19,8 +19,14 @@ namespace {
 #ifndef TXS_CHUNK
 #define TXS_CHUNK 16
 #endif
+#ifndef TXS_CHUNK_BWD_SHORT
+#define TXS_CHUNK_BWD_SHORT 8
+#endif
 #ifndef TXS_BATCH
 #define TXS_BATCH 4
+#endif
+#ifndef TXS_BATCH_BWD
+#define TXS_BATCH_BWD TXS_BATCH
 #endif
 #ifndef TXS_NT_LOADS
 #define TXS_NT_LOADS 1
@@ -30,7 +36,10 @@ namespace {
 #endif
 
 constexpr int kThreads = 256;        // 4 wavefronts per workgroup
-constexpr int kChunk = TXS_CHUNK;    // sorted positions per lane group
+constexpr int kChunk = TXS_CHUNK;    // sorted positions per lane group (forward)
+constexpr int kChunkBwdShort = TXS_CHUNK_BWD_SHORT;  // backward kernel, mean run shorter than kChunkBwdLong
+constexpr int kChunkBwdLong = TXS_CHUNK;             // backward kernel, longer runs
+constexpr int kBatchBwd = TXS_BATCH_BWD;
 constexpr int kBatch = TXS_BATCH;    // rows per load batch of a lane group (two batches in flight)
 constexpr int kHeavyDefault = 64;    // voxels above this many rows use the atomic path
 constexpr int kSpecialBit = (int)0x80000000;
