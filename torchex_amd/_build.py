@@ -7,7 +7,8 @@ cross-compiles for gfx950):
                            compiler against the torch headers; links to the
                            library above through ``$ORIGIN``.
 
-``python -m torchex_amd._build`` builds both.
+``python torchex_amd/_build.py`` builds both (run it as a script: importing the
+package needs the very files this module creates).
 """
 import os
 import subprocess

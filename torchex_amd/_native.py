@@ -12,7 +12,7 @@ KERNEL_LIB = os.path.join(_PKG, "libtorchex_scatter.so")
 
 if not os.path.exists(KERNEL_LIB):
     raise ImportError(
-        f"{KERNEL_LIB} is missing: build it with `python -m torchex_amd._build` "
+        f"{KERNEL_LIB} is missing: build it with `python torchex_amd/_build.py` "
         "(there is no CPU or PyTorch fallback for the scatter kernels)")
 
 try:
@@ -20,7 +20,7 @@ try:
 except ImportError as e:  # pragma: no cover
     raise ImportError(
         "torchex_amd.scatter_ext (the C++ extension module) failed to load: "
-        f"{e}; build it with `python -m torchex_amd._build`") from e
+        f"{e}; build it with `python torchex_amd/_build.py`") from e
 
 # The reference does `import scatter_ext` (torchex/operator_py/scatter_op.py:4);
 # keep that spelling importable.
