@@ -112,7 +112,10 @@ class ScatterData:
 
     def scratch(self, channel):
         """Zeroed table the special voxels are merged in; the kernels leave it
-        zeroed again, so one buffer per channel count is kept for reuse."""
+        zeroed again, so one buffer per channel count is kept for reuse.  Forward
+        calls that share a ``ScatterData`` therefore must not overlap in time on the
+        GPU (two streams running them concurrently would race on this table); calls
+        on one stream, the normal case, are ordered."""
         buf = self._scratch.get(channel)
         if buf is None:
             buf = scatter_ext.make_scratch(self.num_special, channel, self.seg)
