@@ -640,3 +640,56 @@ def test_runs_on_the_current_stream():
         assert torch.equal(mx, ref[0]) and torch.equal(arg, ref[1])
     light = (w.unq_cnts <= data.heavy_threshold).to(DEV)
     assert torch.equal(means[0][light], means[2][light])
+
+
+def test_hip_graph_capture_and_replay():
+    """The forward and backward entry points only launch kernels (no memset node, no
+    host synchronisation, scratch re-zeroed by a kernel), so they can be recorded into
+    a HIP graph.  Every replay is checked against the eager result, with eager work
+    and synchronisations between replays."""
+    from torchex_amd._native import scatter_ext
+    w = workloads.zipf_contention(N=300_000, C=32, num_ids=700, seed=31)   # every voxel on the atomic path
+    w2 = workloads.lidar_sweep(N=200_000, C=64, seed=32)
+    for wl in (w, w2):
+        N, C, U = wl.N, wl.C, wl.U
+        say(f"[case] graph replay {wl.name} N={N} C={C} U={U}")
+        inv, cnts = wl.unq_inv.to(DEV), wl.unq_cnts.to(DEV)
+        f = wl.feats.to(DEV)
+        g = workloads.upstream_grad(U, C, 9).to(DEV)
+        data = tx().ScatterData(inv, cnts)
+        plan = (data.perm, data.seg, data.preSum, data.slot_of, data.heavy_ids, data.scratch(C), data.max_cnt)
+        bplan = (data.perm, data.seg, data.preSum, N)
+
+        def run():
+            mean, _ = scatter_ext.forward(scatter_ext.MEAN, f, *plan)
+            mx, arg = scatter_ext.forward(scatter_ext.MAX, f, *plan)
+            g_mean = scatter_ext.backward(scatter_ext.MEAN, g, None, *bplan)
+            g_max = scatter_ext.backward(scatter_ext.MAX, g, arg, *bplan)
+            return mean, mx, arg, g_mean, g_max
+
+        eager = [t.clone() for t in run()]
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            run()                                   # warm-up on the capture stream
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph):
+            captured = run()
+        light = (wl.unq_cnts <= data.heavy_threshold).to(DEV)
+        for rep in range(3):
+            for t in captured:
+                t.fill_(7)                          # eager work between replays; stale outputs would show
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            mean, mx, arg, g_mean, g_max = captured
+            assert torch.equal(mx, eager[1]) and torch.equal(arg, eager[2]), f"replay {rep}: max"
+            assert torch.equal(g_mean, eager[3]) and torch.equal(g_max, eager[4]), f"replay {rep}: backward"
+            # voxels reduced through atomics may differ in the last bits between runs
+            assert torch.equal(mean[light], eager[0][light]), f"replay {rep}: mean (register path)"
+            assert torch.allclose(mean, eager[0], rtol=1e-5, atol=1e-5, equal_nan=True), f"replay {rep}: mean"
+            # the scratch table is zero again after every replay
+            assert not bool((data.scratch(C) != 0).any()), f"replay {rep}: scratch table not zero"
