@@ -37,9 +37,9 @@ HBM_PEAK_GBPS = 8000.0
 # reads half of the copied bytes on this part: factor 2.000; WRITE_SIZE: factor 1.000).
 MEASURED_TRAFFIC_BYTES = {
     "max_fwd": 525.4e6 + 334.7e6,
-    "max_bwd": 361.9e6 + 512.1e6,
+    "max_bwd": 363.2e6 + 512.2e6,
     "mean_fwd": 525.5e6 + 167.4e6,
-    "mean_bwd": 184.8e6 + 512.0e6,
+    "mean_bwd": 185.3e6 + 512.1e6,
 }
 
 
@@ -304,6 +304,8 @@ def main():
     row_bytes = C * esz
     vec = next(v for v in (16, 8, 4, 2) if row_bytes % v == 0 and v >= esz) // esz   # elements per lane
     kname = "scatter_%s_kernel<%s,%d,%s>" % (dom[-3:], a.dtype.upper(), vec, dom[:-4].upper())
+    if dom.endswith("bwd"):   # the backward kernel also carries its chunk (positions per lane group)
+        kname = kname[:-1] + (",8>" if N < 16 * U else ",16>")
     roofline = {"bound": "hbm", "kernel": kname, "achieved": per_kernel[dom]["GBps"], "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s", "frac": per_kernel[dom]["frac"],
                 "traffic": MEASURED_TRAFFIC_BYTES[dom]
