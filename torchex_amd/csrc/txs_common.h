@@ -66,11 +66,9 @@ struct BF16 {
     static __device__ __forceinline__ float to_f(raw x) {
         return __uint_as_float(((unsigned)x) << 16);
     }
-    static __device__ __forceinline__ raw from_f(float x) {  // round to nearest even
-        unsigned b = __float_as_uint(x);
-        if ((b & 0x7fffffffu) > 0x7f800000u) return (raw)((b >> 16) | 0x0040u);
-        b += 0x7fffu + ((b >> 16) & 1u);
-        return (raw)(b >> 16);
+    static __device__ __forceinline__ raw from_f(float x) {
+        // round to nearest even in hardware (v_cvt_pk_bf16_f32 on gfx950); NaN stays NaN
+        return __builtin_bit_cast(unsigned short, (__bf16)x);
     }
     static __device__ __forceinline__ raw lowest() { return (raw)0xff7f; }
     static __device__ __forceinline__ raw zero() { return (raw)0; }
