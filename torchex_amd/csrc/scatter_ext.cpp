@@ -356,6 +356,7 @@ Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const 
     TORCH_CHECK(grad_out.size(0) == U, "grad_out has ", grad_out.size(0), " rows, plan has ", U, " voxels");
     TORCH_CHECK(seg.numel() == N, "plan row count mismatch");
     TORCH_CHECK(!perm.has_value() || perm->numel() == N, "perm length mismatch");
+    TORCH_CHECK(seg.device() == grad_out.device(), "plan and grad_out live on different devices");
     if (op == TXS_MAX || op == TXS_MAX_REFTIE) {
         TORCH_CHECK(arg.has_value(), "scatter_max backward needs arg");
         check_i32(*arg, "arg");
