@@ -693,3 +693,32 @@ def test_hip_graph_capture_and_replay():
             assert torch.allclose(mean, eager[0], rtol=1e-5, atol=1e-5, equal_nan=True), f"replay {rep}: mean"
             # the scratch table is zero again after every replay
             assert not bool((data.scratch(C) != 0).any()), f"replay {rep}: scratch table not zero"
+
+
+def test_random_small_shapes_sweep():
+    """Seeded sweep over small random problems: row counts, channel widths, voxel counts,
+    occupancy profiles (uniform, skewed, with empty voxels, grouped or shuffled) and
+    heavy thresholds, each checked like every other case (plan, forward, backward)."""
+    rs = np.random.RandomState(1234)
+    for case in range(60):
+        N = int(rs.choice([1, 2, 7, 15, 16, 17, 63, 64, 65, 129, 500, 1023, 2049, 4000]))
+        C = int(rs.choice([1, 2, 3, 4, 5, 8, 12, 16, 31, 32, 33, 64, 100, 128]))
+        U = int(rs.randint(1, N + 1))
+        kind = case % 4
+        if kind == 0:      # uniform ids (some voxels may stay empty)
+            ids = rs.randint(0, U, size=N)
+        elif kind == 1:    # skewed: most rows in a few voxels
+            ids = np.minimum((rs.exponential(scale=max(U / 8.0, 1.0), size=N)).astype(np.int64), U - 1)
+        elif kind == 2:    # one long run plus singletons
+            ids = np.concatenate([np.zeros(N - N // 3, dtype=np.int64), rs.randint(0, U, size=N // 3)])
+        else:              # every id at least once where possible
+            ids = np.concatenate([np.arange(min(U, N)), rs.randint(0, U, size=N - min(U, N))])
+        ids = np.sort(ids) if case % 3 == 0 else rs.permutation(ids)
+        inv = torch.from_numpy(ids.astype(np.int64))
+        cnts = torch.bincount(inv, minlength=U)
+        feats = torch.from_numpy(rs.standard_normal((N, C)).astype(np.float32))
+        if case % 5 == 0:  # plant ties
+            feats = torch.round(feats * 2) / 2
+        thr = int(rs.choice([16, 17, 33, 64]))
+        dtype = [torch.float32, torch.float32, torch.float16, torch.bfloat16][case % 4] if case % 2 else torch.float32
+        run_case(f"sweep{case}", feats, inv, cnts, dtype=dtype, grad_seed=case, heavy_threshold=thr)
