@@ -722,3 +722,26 @@ def test_random_small_shapes_sweep():
         thr = int(rs.choice([16, 17, 33, 64]))
         dtype = [torch.float32, torch.float32, torch.float16, torch.bfloat16][case % 4] if case % 2 else torch.float32
         run_case(f"sweep{case}", feats, inv, cnts, dtype=dtype, grad_seed=case, heavy_threshold=thr)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_subnormal_values_are_kept(dtype):
+    """Subnormal inputs are neither flushed on the way in nor on the way out (the
+    output conversion of bf16 is a hardware instruction): max returns them bit for
+    bit and a two-term sum equals the correctly rounded fp32 sum."""
+    T = tx()
+    tiny = {torch.float32: [1e-40, -3e-41, 2e-39, 5e-45],
+            torch.bfloat16: [1e-40, -3e-41, 2e-39, 5e-45],
+            torch.float16: [6e-8, -2e-7, 3e-6, 1e-7]}[dtype]
+    v = torch.tensor(tiny, dtype=torch.float32).to(dtype)
+    f = v.reshape(4, 1).repeat(1, 8).to(DEV)
+    data = T.ScatterData(torch.tensor([0, 0, 1, 1], device=DEV), torch.tensor([2, 2], device=DEV))
+    mx, arg = T.scatter_max(f, data)
+    s = T.scatter_sum(f, data)
+    want_max = torch.stack([torch.maximum(v[0], v[1]), torch.maximum(v[2], v[3])])
+    want_sum = torch.stack([(v[0].float() + v[1].float()).to(dtype), (v[2].float() + v[3].float()).to(dtype)])
+    for c in range(8):
+        assert torch.equal(mx[:, c].cpu().view(torch.int16 if dtype != torch.float32 else torch.int32),
+                           want_max.view(torch.int16 if dtype != torch.float32 else torch.int32))
+        assert torch.equal(s[:, c].cpu().float(), want_sum.float())
+    assert float(want_max.float().abs().min()) > 0.0   # the case really holds subnormals, not zeros
