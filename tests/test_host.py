@@ -29,6 +29,28 @@ def test_header_symbols_are_exported():
     assert not missing, missing
 
 
+def test_header_is_plain_c_and_links(tmp_path):
+    """The boundary is a C ABI: the header compiles as C11 with no extensions and a C
+    program links against the library without any C++ or torch symbol in sight."""
+    import shutil
+    import subprocess
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        import pytest
+        pytest.skip("no C compiler on this machine")
+    src = tmp_path / "abi.c"
+    src.write_text('#include "torchex_scatter.h"\n'
+                   'int main(void) { return txs_abi_version() == 5 && txs_chunk_rows() > 0 ? 0 : 1; }\n')
+    inc = os.path.join(ROOT, "include")
+    pkg = os.path.join(ROOT, "torchex_amd")
+    subprocess.check_call([cc, "-std=c11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I" + inc,
+                           "-fsyntax-only", str(src)])
+    exe = tmp_path / "abi"
+    subprocess.check_call([cc, "-std=c11", "-I" + inc, str(src), "-L" + pkg, "-ltorchex_scatter",
+                           "-Wl,-rpath," + pkg, "-o", str(exe)])
+    assert subprocess.call([str(exe)]) == 0
+
+
 def test_host_only_entry_points():
     lib = _lib()
     assert lib.txs_abi_version() == 5
