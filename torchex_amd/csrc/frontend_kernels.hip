@@ -260,8 +260,13 @@ __global__ __launch_bounds__(kThreads) void dpp_write_kernel(
 // them out) claimed with a single 64-bit compare-and-swap, so key and value
 // appear together.
 
-__device__ __forceinline__ int grid_hash_slot(long long key, int probe_i, int table_size) {
-    return (int)((key % table_size + probe_i * (key * 2 + 1)) % table_size);
+// (key % size + i * (2 * key + 1)) % size of the reference, for key >= 0 and a
+// power-of-two size: both remainders are bit masks and the 64-bit sum cannot wrap
+// (i < size <= 2^30, 2 * key + 1 < 2^32).
+__device__ __forceinline__ int grid_hash_slot(int key, int probe_i, int table_size) {
+    const unsigned long long mask = (unsigned long long)(table_size - 1);
+    const unsigned long long k = (unsigned long long)(unsigned)key;
+    return (int)(((k & mask) + (unsigned long long)probe_i * (k * 2ull + 1ull)) & mask);
 }
 
 __global__ void grid_hash_build_kernel(const int *__restrict__ keys, const int *__restrict__ values,
@@ -273,9 +278,8 @@ __global__ void grid_hash_build_kernel(const int *__restrict__ keys, const int *
     const unsigned long long word =
         ((unsigned long long)(unsigned)values[i] << 32) | (unsigned long long)(unsigned)key;
     const unsigned long long empty = ~0ull;  // (-1, -1)
-    for (int t = 0; t < table_size; ++t) {
+    for (int t = 0; key >= 0 && t < table_size; ++t) {
         const int s = grid_hash_slot(key, t, table_size);
-        if ((unsigned)s >= (unsigned)table_size) break;  // negative key
         if (atomicCAS(table + s, empty, word) == empty) return;
     }
     if (fail) fail[0] = 1;  // table full or key negative (the reference asserts)
@@ -288,9 +292,8 @@ __global__ void grid_hash_probe_kernel(const int *__restrict__ keys,
     if (i >= n) return;
     const int key = keys[i];
     int v = -1;
-    for (int t = 0; t < table_size; ++t) {
+    for (int t = 0; key >= 0 && t < table_size; ++t) {
         const int s = grid_hash_slot(key, t, table_size);
-        if ((unsigned)s >= (unsigned)table_size) break;
         const unsigned long long word = table[s];
         const int slot_key = (int)(unsigned)(word & 0xffffffffull);
         if (slot_key == key) {
