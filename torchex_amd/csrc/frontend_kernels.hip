@@ -120,6 +120,7 @@ constexpr int kDppInfo = 13;
 
 struct DppBox {
     float cx, cy, czc, w, l, h, cosa, sina, large_w, large_l, large_h, cz_bottom;
+    float r2;  // squared radius of a circle around (cx, cy) that contains the box and its margin
 };
 
 // per-box constants, computed once so both passes see identical numbers; the
@@ -143,7 +144,18 @@ __global__ void dpp_box_kernel(const float *__restrict__ rois, int B, float extr
     const float rot = (float)((double)r[6] + 3.14159265358979323846 / 2);  // (:24)
     bx.cosa = (float)cos((double)rot);
     bx.sina = (float)sin((double)rot);
+    // generous bound (0.1 % + 1 mm^2): a point outside this circle fails the exact
+    // test whatever the rounding, so skipping it cannot change the result
+    const float hl = 0.5f * fmaxf(fabsf(bx.l), fabsf(bx.large_l));
+    const float hw = 0.5f * fmaxf(fabsf(bx.w), fabsf(bx.large_w));
+    bx.r2 = (hl * hl + hw * hw) * 1.001f + 1e-6f;
     boxes[b] = bx;
+}
+
+// cheap conservative reject in the xy plane; most waves skip the exact test with it
+__device__ __forceinline__ bool dpp_near(const DppBox &bx, float x, float y) {
+    const float sx = x - bx.cx, sy = y - bx.cy;
+    return sx * sx + sy * sy <= bx.r2;
 }
 
 // 0: outside the enlarged box, 1: in the margin, 2: inside the box (:33-71)
@@ -163,26 +175,39 @@ __device__ __forceinline__ int dpp_test(const DppBox &bx, float x, float y, floa
     return in_box ? 2 : (in_large ? 1 : 0);
 }
 
-// hits per (box, tile); grid (tiles, boxes)
+// A workgroup keeps its 256 points in registers and walks kDppBoxesPerWg boxes, so the
+// points are read once per group of boxes and the box constants come through the
+// scalar path.
+constexpr int kDppBoxesPerWg = 8;
+
+// hits per (box, tile); grid (tiles, groups of boxes)
 __global__ __launch_bounds__(kThreads) void dpp_count_kernel(const float *__restrict__ pts, int P,
-                                                             const DppBox *__restrict__ boxes,
+                                                             const DppBox *__restrict__ boxes, int B,
                                                              int n_tiles, int *__restrict__ counts) {
-    __shared__ int wsum[kThreads / 64];
+    __shared__ int cnt[kDppBoxesPerWg];
     const int p = blockIdx.x * kThreads + threadIdx.x;
-    const DppBox bx = boxes[blockIdx.y];
-    bool hit = false;
-    if (p < P) {
-        float lx, ly;
-        hit = dpp_test(bx, pts[(size_t)p * 3], pts[(size_t)p * 3 + 1], pts[(size_t)p * 3 + 2], lx, ly) > 0;
-    }
-    const int c = __popcll(__ballot(hit));
-    if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = c;
+    const int b0 = blockIdx.y * kDppBoxesPerWg;
+    if (threadIdx.x < kDppBoxesPerWg) cnt[threadIdx.x] = 0;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int t = 0;
-        for (int k = 0; k < kThreads / 64; ++k) t += wsum[k];
-        counts[(size_t)blockIdx.y * n_tiles + blockIdx.x] = t;
+    float x = 0.f, y = 0.f, z = 0.f;
+    if (p < P) {
+        x = pts[(size_t)p * 3];
+        y = pts[(size_t)p * 3 + 1];
+        z = pts[(size_t)p * 3 + 2];
     }
+    for (int bb = 0; bb < kDppBoxesPerWg && b0 + bb < B; ++bb) {
+        const DppBox bx = boxes[b0 + bb];
+        bool hit = false;
+        if (p < P && dpp_near(bx, x, y)) {
+            float lx, ly;
+            hit = dpp_test(bx, x, y, z, lx, ly) > 0;
+        }
+        const int c = __popcll(__ballot(hit));
+        if (c && (threadIdx.x & 63) == 0) atomicAdd(&cnt[bb], c);
+    }
+    __syncthreads();
+    if (threadIdx.x < kDppBoxesPerWg && b0 + (int)threadIdx.x < B)
+        counts[(size_t)(b0 + threadIdx.x) * n_tiles + blockIdx.x] = cnt[threadIdx.x];
 }
 
 // per-box kept count = min(hits, cap), exclusive scan over boxes, total (one workgroup)
@@ -205,51 +230,69 @@ __global__ __launch_bounds__(kThreads) void dpp_box_base_kernel(const int *__res
 
 // second pass: same test, rank of the hit inside its box, compact write
 __global__ __launch_bounds__(kThreads) void dpp_write_kernel(
-    const float *__restrict__ pts, int P, const DppBox *__restrict__ boxes, int n_tiles,
+    const float *__restrict__ pts, int P, const DppBox *__restrict__ boxes, int B, int n_tiles,
     const int *__restrict__ scanned, const int *__restrict__ box_base, int cap, int max_all,
     long long *__restrict__ out_pts_idx, long long *__restrict__ out_roi_idx,
     float *__restrict__ out_feats) {
 #pragma clang fp contract(off)
-    __shared__ int wsum[kThreads / 64];
-    const int b = blockIdx.y;
+    __shared__ int wsum[kDppBoxesPerWg][kThreads / 64];
+    const int b0 = blockIdx.y * kDppBoxesPerWg;
     const int p = blockIdx.x * kThreads + threadIdx.x;
-    const DppBox bx = boxes[b];
-    int flag = 0;
-    float x = 0.f, y = 0.f, z = 0.f, lx = 0.f, ly = 0.f;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    float x = 0.f, y = 0.f, z = 0.f;
     if (p < P) {
         x = pts[(size_t)p * 3];
         y = pts[(size_t)p * 3 + 1];
         z = pts[(size_t)p * 3 + 2];
-        flag = dpp_test(bx, x, y, z, lx, ly);
     }
-    const unsigned long long m = __ballot(flag > 0);
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    if (lane == 0) wsum[w] = __popcll(m);
+    // phase 1: the test against every box of the group (2 result bits per box) and the
+    // hits of each wave
+    unsigned flags = 0u;
+    for (int bb = 0; bb < kDppBoxesPerWg && b0 + bb < B; ++bb) {
+        const DppBox bx = boxes[b0 + bb];
+        int flag = 0;
+        if (p < P && dpp_near(bx, x, y)) {
+            float lx, ly;
+            flag = dpp_test(bx, x, y, z, lx, ly);
+        }
+        flags |= (unsigned)flag << (2 * bb);
+        const unsigned long long m = __ballot(flag > 0);
+        if (lane == 0) wsum[bb][w] = __popcll(m);
+    }
     __syncthreads();
-    if (flag == 0) return;
-    int rank = __popcll(m & ((1ull << lane) - 1ull));
-    for (int k = 0; k < w; ++k) rank += wsum[k];
-    rank += scanned[(size_t)b * n_tiles + blockIdx.x] - scanned[(size_t)b * n_tiles];
-    if (rank >= cap) return;
-    const long pos = (long)box_base[b] + rank;
-    if (pos >= max_all) return;
-    const float local_z = (float)((double)z - ((double)bx.cz_bottom + (double)bx.h / 2.0));  // (:103)
-    float *f = out_feats + pos * kDppInfo;
-    out_pts_idx[pos] = p;
-    out_roi_idx[pos] = b;
-    f[0] = x;
-    f[1] = y;
-    f[2] = z;
-    f[3] = lx;
-    f[4] = ly;
-    f[5] = local_z;
-    f[6] = lx + bx.l / 2;
-    f[7] = ly + bx.w / 2;
-    f[8] = local_z + bx.h / 2;
-    f[9] = -lx + bx.l / 2;
-    f[10] = -ly + bx.w / 2;
-    f[11] = -local_z + bx.h / 2;
-    f[12] = flag == 1 ? 1.0f : 0.0f;
+    // phase 2: rank of each hit inside its box, compact write (hits are rare)
+    for (int bb = 0; bb < kDppBoxesPerWg && b0 + bb < B; ++bb) {
+        const int flag = (int)((flags >> (2 * bb)) & 3u);
+        const unsigned long long m = __ballot(flag > 0);
+        if (flag == 0) continue;
+        const int b = b0 + bb;
+        int rank = __popcll(m & ((1ull << lane) - 1ull));
+        for (int k = 0; k < w; ++k) rank += wsum[bb][k];
+        rank += scanned[(size_t)b * n_tiles + blockIdx.x] - scanned[(size_t)b * n_tiles];
+        if (rank >= cap) continue;
+        const long pos = (long)box_base[b] + rank;
+        if (pos >= max_all) continue;
+        const DppBox bx = boxes[b];
+        float lx, ly;
+        dpp_test(bx, x, y, z, lx, ly);  // the same arithmetic as in phase 1
+        const float local_z = (float)((double)z - ((double)bx.cz_bottom + (double)bx.h / 2.0));  // (:103)
+        float *f = out_feats + pos * kDppInfo;
+        out_pts_idx[pos] = p;
+        out_roi_idx[pos] = b;
+        f[0] = x;
+        f[1] = y;
+        f[2] = z;
+        f[3] = lx;
+        f[4] = ly;
+        f[5] = local_z;
+        f[6] = lx + bx.l / 2;
+        f[7] = ly + bx.w / 2;
+        f[8] = local_z + bx.h / 2;
+        f[9] = -lx + bx.l / 2;
+        f[10] = -ly + bx.w / 2;
+        f[11] = -local_z + bx.h / 2;
+        f[12] = flag == 1 ? 1.0f : 0.0f;
+    }
 }
 
 // ------------------------------------------------------------- grid hash --
@@ -391,12 +434,13 @@ int txs_dynamic_point_pool(const float *rois, const float *pts, int64_t num_boxe
     int *box_base = scan_ws + scan_tiles(cells + 2) + 1;
     dpp_box_kernel<<<dim3(blocks_for(B)), dim3(kThreads), 0, st>>>(rois, B, extra_wlh[0], extra_wlh[1],
                                                                  extra_wlh[2], boxes);
-    dpp_count_kernel<<<dim3(n_tiles, B), dim3(kThreads), 0, st>>>(pts, P, boxes, n_tiles, counts);
+    const int box_groups = (B + kDppBoxesPerWg - 1) / kDppBoxesPerWg;
+    dpp_count_kernel<<<dim3(n_tiles, box_groups), dim3(kThreads), 0, st>>>(pts, P, boxes, B, n_tiles, counts);
     if (exclusive_scan(counts, cells, counts, cells + 1, scan_ws, st) != hipSuccess) return TXS_ERR_LAUNCH;
     dpp_box_base_kernel<<<dim3(1), dim3(kThreads), 0, st>>>(counts, B, n_tiles, max_pts_per_box,
                                                            (int)max_all_pts, box_base, num_out);
-    dpp_write_kernel<<<dim3(n_tiles, B), dim3(kThreads), 0, st>>>(
-        pts, P, boxes, n_tiles, counts, box_base, max_pts_per_box, (int)max_all_pts,
+    dpp_write_kernel<<<dim3(n_tiles, box_groups), dim3(kThreads), 0, st>>>(
+        pts, P, boxes, B, n_tiles, counts, box_base, max_pts_per_box, (int)max_all_pts,
         (long long *)out_pts_idx, (long long *)out_roi_idx, out_pts_feats);
     return status_of(hipGetLastError());
 }
