@@ -191,6 +191,39 @@ def test_dynamic_point_pool(B, P, cap, max_all, extra):
     assert idx.shape[0] <= max_all and torch.bincount(roi).max().item() <= cap
 
 
+def test_dynamic_point_pool_corner_points():
+    """Points placed a hair inside and outside the corners and edge midpoints of the
+    rotated (enlarged) boxes: the farthest places from a box centre that still count,
+    i.e. where a too tight early reject would lose hits.  Includes shrinking margins."""
+    T = tx()
+    g = torch.Generator().manual_seed(17)
+    B = 64
+    rois = torch.zeros((B, 7))
+    rois[:, 0:2] = torch.rand((B, 2), generator=g) * 60 - 30
+    rois[:, 3:6] = torch.rand((B, 3), generator=g) * 6 + 0.5
+    rois[:, 6] = torch.rand((B,), generator=g) * 6.283 - 3.1415
+    for extra in ([0.0, 0.0, 0.0], [0.6, 0.4, 0.2], [-0.2, -0.1, 0.0]):
+        ex = torch.tensor(extra)
+        pts = []
+        for b in range(B):
+            cx, cy, zb, w, l, h, rz = rois[b].tolist()
+            rot = rz + np.pi / 2
+            c, s_ = np.cos(rot), np.sin(rot)
+            for dims in ((l, w), (l + extra[1], w + extra[0])):
+                for ux, uy in ((1, 1), (1, -1), (-1, 1), (-1, -1), (1, 0), (0, 1), (-1, 0), (0, -1)):
+                    for scale in (1 - 1e-6, 1 - 1e-4, 1 + 1e-6, 1 + 1e-4):
+                        lx, ly = ux * dims[0] / 2 * scale, uy * dims[1] / 2 * scale
+                        # inverse of the local transform: world = centre + R^T (lx, ly)
+                        pts.append([cx + lx * c + ly * s_, cy - lx * s_ + ly * c, zb + h / 2])
+        pts = torch.tensor(pts, dtype=torch.float32)
+        say(f"[case] dynamic_point_pool corners extra={extra} P={pts.shape[0]}")
+        idx, roi, feats = T.dynamic_point_pool(rois.to(DEV), pts.to(DEV), extra, 100_000, 1_000_000)
+        wi, wr, wf = orc.dynamic_point_pool(rois.numpy(), pts.numpy(), extra, 100_000, 1_000_000)
+        assert wi.shape[0] > B * 8     # the inner copies are hits
+        assert np.array_equal(idx.cpu().numpy(), wi) and np.array_equal(roi.cpu().numpy(), wr)
+        assert np.array_equal(feats.cpu().numpy().view(np.uint32), wf.view(np.uint32))
+
+
 def test_dynamic_point_pool_no_hits_returns_the_reference_placeholder():
     T = tx()
     rois = torch.tensor([[1000.0, 1000.0, 0.0, 2.0, 4.0, 1.5, 0.3]], device=DEV)
