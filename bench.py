@@ -97,14 +97,21 @@ def cpu_baseline(w, g_mean, g_max):
         tor.step_mean_max(w.feats, w.unq_inv, w.unq_cnts, g_mean, g_max)
         iters += 1
     dt = (time.perf_counter() - t0) / iters
-    return {"value": 2 * w.N / dt, "unit": "points/s", "cores": torch.get_num_threads(),
-            "kind": "port", "ms_per_step": dt * 1e3,
-            "sample": f"{iters} full steps (N={w.N}, C={w.C}) of torch.scatter_reduce/index_add/gather on CPU"}
+    used = torch.get_num_threads()
+    torch.set_num_threads(1)          # one step on a single core, for scale
+    t1 = time.perf_counter()
+    tor.step_mean_max(w.feats, w.unq_inv, w.unq_cnts, g_mean, g_max)
+    dt1 = time.perf_counter() - t1
+    torch.set_num_threads(used)
+    return {"value": 2 * w.N / dt, "unit": "points/s", "cores": used,
+            "kind": "port", "ms_per_step": dt * 1e3, "single_thread_ms_per_step": dt1 * 1e3,
+            "sample": f"{iters} full steps (N={w.N}, C={w.C}) of torch.scatter_reduce/index_add/gather on CPU "
+                      f"with {used} threads, then 1 step with 1 thread"}
 
 
 def instrumented_steps(scatter_ext, f, g_mean, g_max, plan, bplan, steps, warmup):
-    """Average duration (ms) of each of the step's four entry-point calls, issued in step
-    order with a HIP event between them."""
+    """Duration (ms) of each of the step's four entry-point calls, issued in step order with
+    a HIP event between them: (mean per call, {median, min} per call)."""
     names = ("mean_fwd", "mean_bwd", "max_fwd", "max_bwd")
 
     def raw_step(ev=None):
@@ -126,7 +133,10 @@ def instrumented_steps(scatter_ext, f, g_mean, g_max, plan, bplan, steps, warmup
     for e in evs:
         raw_step(e)
     torch.cuda.synchronize()
-    return {n: sum(e[i].elapsed_time(e[i + 1]) for e in evs) / len(evs) for i, n in enumerate(names)}
+    per = {n: sorted(e[i].elapsed_time(e[i + 1]) for e in evs) for i, n in enumerate(names)}
+    mean = {n: sum(v) / len(v) for n, v in per.items()}
+    spread = {n: {"median_ms": v[len(v) // 2], "min_ms": v[0]} for n, v in per.items()}
+    return mean, spread
 
 
 def frontend_timings(T, workloads, dev, N):
@@ -253,7 +263,7 @@ def main():
     plan = (data.perm, data.seg, data.preSum, data.slot_of, data.heavy_ids, sc, data.max_cnt)
     bplan = (data.perm, data.seg, data.preSum, N)
     _, arg = scatter_ext.forward(scatter_ext.MAX, f, *plan)
-    kt = instrumented_steps(scatter_ext, f, g_mean, g_max, plan, bplan, a.steps, a.warmup)
+    kt, kt_spread = instrumented_steps(scatter_ext, f, g_mean, g_max, plan, bplan, a.steps, a.warmup)
     kernel_sum_ms = sum(kt.values())
 
     # the same points delivered grouped by voxel, which is the only order the reference's
@@ -265,8 +275,8 @@ def main():
         data_s = T.ScatterData(inv[order].contiguous(), cnts)
         plan_s = (data_s.perm, data_s.seg, data_s.preSum, data_s.slot_of, data_s.heavy_ids,
                   data_s.scratch(C), data_s.max_cnt)
-        kts = instrumented_steps(scatter_ext, f_s, g_mean, g_max, plan_s,
-                                 (data_s.perm, data_s.seg, data_s.preSum, N), a.steps, a.warmup)
+        kts, _ = instrumented_steps(scatter_ext, f_s, g_mean, g_max, plan_s,
+                                    (data_s.perm, data_s.seg, data_s.preSum, N), a.steps, a.warmup)
         sorted_input = {"per_kernel_ms": kts, "kernel_sum_ms": sum(kts.values()),
                         "points_per_s": 2 * N / sum(kts.values()) * 1e3}
         del f_s, data_s, plan_s, order
@@ -286,7 +296,8 @@ def main():
             "max_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MAX, g_max, arg, *bplan), it),
         }
     ab = {k: workloads.algorithmic_bytes(k, N, C, U, esz) for k in kt}
-    per_kernel = {k: {"ms": kt[k], "GBps": ab[k] / kt[k] / 1e6, "frac": ab[k] / kt[k] / 1e6 / HBM_PEAK_GBPS}
+    per_kernel = {k: {"ms": kt[k], "GBps": ab[k] / kt[k] / 1e6, "frac": ab[k] / kt[k] / 1e6 / HBM_PEAK_GBPS,
+                      **kt_spread.get(k, {})}
                   for k in kt}
     per_op = {}
     for op in ("mean", "max", "sum"):
