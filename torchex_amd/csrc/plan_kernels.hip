@@ -65,6 +65,7 @@ __global__ void presum_from_sorted_kernel(const int *__restrict__ keys, long n, 
 
 constexpr int kScanItems = 8;
 constexpr int kScanTile = kThreads * kScanItems;
+constexpr int kScanFusedTiles = 1024;  // up to this many tiles the apply kernel sums the tile totals itself
 
 __global__ __launch_bounds__(kThreads) void scan_tile_sums_kernel(const int *__restrict__ in,
                                                                   long n_in,
@@ -94,9 +95,13 @@ __global__ __launch_bounds__(kThreads) void scan_tile_offsets_kernel(int *__rest
     }
 }
 
-// in and out may be the same array: a thread reads its items before any write
+// in and out may be the same array: a thread reads its items before any write.
+// With offsets_ready == 0, tile_offs still holds the plain tile sums and the
+// workgroup adds up the ones in front of its own tile itself (cheaper than a
+// launch of its own while there are few tiles).
 __global__ __launch_bounds__(kThreads) void scan_apply_kernel(const int *in, long n_in, int *out,
-                                                              long n_out, const int *tile_offs) {
+                                                              long n_out, const int *tile_offs,
+                                                              int offsets_ready) {
     long base = (long)blockIdx.x * kScanTile + (long)threadIdx.x * kScanItems;
     int x[kScanItems];
     int s = 0;
@@ -106,8 +111,16 @@ __global__ __launch_bounds__(kThreads) void scan_apply_kernel(const int *in, lon
         x[k] = (i < n_in) ? in[i] : 0;
         s += x[k];
     }
+    int tile_off;
+    if (offsets_ready) {
+        tile_off = tile_offs[blockIdx.x];
+    } else {
+        int part = 0;
+        for (int t = threadIdx.x; t < (int)blockIdx.x; t += kThreads) part += tile_offs[t];
+        block_exclusive_scan(part, &tile_off);
+    }
     int tot;
-    int run = block_exclusive_scan(s, &tot) + tile_offs[blockIdx.x];
+    int run = block_exclusive_scan(s, &tot) + tile_off;
 #pragma unroll
     for (int k = 0; k < kScanItems; ++k) {
         long i = base + k;
@@ -127,8 +140,9 @@ hipError_t exclusive_scan(const int *in, long n_in, int *out, long n_out, int *w
     if (n_out <= 0) return hipSuccess;
     long tiles = scan_tiles(n_out);
     scan_tile_sums_kernel<<<dim3((unsigned)tiles), dim3(kThreads), 0, st>>>(in, n_in, ws);
-    scan_tile_offsets_kernel<<<dim3(1), dim3(kThreads), 0, st>>>(ws, tiles);
-    scan_apply_kernel<<<dim3((unsigned)tiles), dim3(kThreads), 0, st>>>(in, n_in, out, n_out, ws);
+    const int few = tiles <= kScanFusedTiles;
+    if (!few) scan_tile_offsets_kernel<<<dim3(1), dim3(kThreads), 0, st>>>(ws, tiles);
+    scan_apply_kernel<<<dim3((unsigned)tiles), dim3(kThreads), 0, st>>>(in, n_in, out, n_out, ws, !few);
     return hipGetLastError();
 }
 
