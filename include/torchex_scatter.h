@@ -21,11 +21,13 @@
  *                       non-decreasing (position == row)
  *   seg        [N]      int32 voxel id at each sorted position, bit 31 set when
  *                       the voxel is "special" (see below)
- *   slot_of    [U]      int32 slot of a special voxel in heavy_ids/scratch, else -1
- *   heavy_ids  [>=n_special] int32 voxel id per slot
- *   scratch    [n_special * C] 8-byte cells.  MUST BE ZERO ON ENTRY to
- *                       txs_scatter_forward and is zero again when the call's
- *                       kernels have finished.
+ *   slot_of    [U]      int32 >= 0 for a special voxel (for a heavy one: its slot
+ *                       in heavy_ids and its row in scratch), else -1
+ *   heavy_ids  [n_special] int32 ids of the special voxels, the n_heavy heavy
+ *                       ones first (slot order), the empty ones after them
+ *   scratch    [n_heavy * C] 8-byte cells, one row per heavy voxel.  MUST BE
+ *                       ZERO ON ENTRY to txs_scatter_forward and is zero again
+ *                       when the call's kernels have finished.
  *   out        [U, C]   dtype of feats;  arg [U, C] int32 (row index into feats)
  *
  * Special voxels: a voxel with more than `heavy_threshold` rows is reduced by
@@ -57,6 +59,7 @@ enum {
     TXS_STAT_NUM_EMPTY = 4,    /* number of voxels with zero rows */
     TXS_STAT_COUNT_MISMATCH = 5, /* 1 if the caller's unq_cnts is not the histogram of unq_inv */
     TXS_STAT_NUM_UNQ = 6,      /* number of distinct keys found by txs_unique_runs */
+    TXS_STAT_NUM_HEAVY = 7,    /* number of voxels above the heavy threshold (NUM_SPECIAL - NUM_EMPTY) */
     TXS_STATS_LEN = 8
 };
 
@@ -107,10 +110,12 @@ int txs_plan_presum(const int32_t *sorted_keys, int64_t num_total, int64_t num_u
                     int32_t *preSum, void *stream);
 
 /* Table of special voxels (heavy or empty) from CSR offsets, stats[MAX_CNT],
- * stats[NUM_SPECIAL], stats[NUM_EMPTY]; when unq_cnts (int64 [num_unq], as
+ * stats[NUM_SPECIAL], stats[NUM_HEAVY], stats[NUM_EMPTY]; when unq_cnts (int64 [num_unq], as
  * torch.unique returns it) is given, stats[COUNT_MISMATCH] is set if it is not
  * the histogram of unq_inv (the consistency check of scatter_op.py:19).
- * heavy_ids must hold num_unq entries (the first NUM_SPECIAL are used).
+ * heavy_ids must hold num_unq entries: on return its first NUM_HEAVY entries
+ * are the heavy voxels and its LAST NUM_EMPTY entries the empty ones; the list
+ * txs_scatter_forward takes is those two pieces put together, heavy first.
  * num_unq_dev (may be NULL): device int holding the true voxel count when the
  * host only knows the upper bound passed as num_unq (after txs_unique_runs).
  * cnts_out (may be NULL): int64 [num_unq] voxel populations, the unq_cnts of
@@ -214,7 +219,7 @@ int txs_grid_hash_probe(const int32_t *keys, int64_t num_keys, const int32_t *ta
  *     -inf never wins, as in the reference.  max_cnt is the largest voxel
  *     population (the reference launcher's argument); other ops ignore it.
  * out (and arg) need no initialisation: every element is written.
- * scratch may be NULL when num_special == 0. */
+ * scratch may be NULL when there is no heavy voxel (empty voxels need none). */
 int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *perm,
                         const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
                         const int32_t *heavy_ids, int64_t num_special, void *scratch,

@@ -745,3 +745,21 @@ def test_subnormal_values_are_kept(dtype):
                            want_max.view(torch.int16 if dtype != torch.float32 else torch.int32))
         assert torch.equal(s[:, c].cpu().float(), want_sum.float())
     assert float(want_max.float().abs().min()) > 0.0   # the case really holds subnormals, not zeros
+
+
+def test_mostly_empty_voxel_grid():
+    """Ids scattered over a large dense grid: a million voxels, almost all empty, one
+    heavy.  Empty voxels get their rows without owning scratch memory (one scratch row
+    per heavy voxel only), and slot allocation does not queue on one counter."""
+    U, N, C = 1_000_000, 30_000, 8
+    g = torch.Generator().manual_seed(77)
+    inv = torch.randint(0, U, (N,), generator=g)
+    inv[:500] = 123_456                      # one voxel above the heavy threshold
+    cnts = torch.bincount(inv, minlength=U)
+    feats = torch.randn((N, C), generator=g)
+    data = run_case("mostly_empty", feats, inv, cnts)
+    assert data.num_heavy == 1 and data.num_special == int((cnts == 0).sum()) + 1
+    assert tuple(data.scratch(C).shape) == (1, C)
+    # layout the kernels rely on: heavy voxels first, then the empty ones
+    ids = data.heavy_ids.cpu()
+    assert ids[0].item() == 123_456 and bool((cnts[ids[1:].long()] == 0).all())

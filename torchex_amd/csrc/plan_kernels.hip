@@ -170,40 +170,55 @@ __global__ __launch_bounds__(kSpecialThreads) void plan_special_kernel(
     const long long *__restrict__ unq_cnts, int *__restrict__ slot_of,
     int *__restrict__ heavy_ids, int *__restrict__ stats, const int *__restrict__ num_unq_dev,
     long long *__restrict__ cnts_out) {
-    __shared__ int s_max[kSpecialThreads / 64], s_empty[kSpecialThreads / 64], s_bad[kSpecialThreads / 64];
+    __shared__ int s_max[kSpecialThreads / 64], s_bad[kSpecialThreads / 64];
     // the voxel count may only be known on the device (unique path): U_arg is then an upper bound
     const int U = num_unq_dev ? min(U_arg, *num_unq_dev) : U_arg;
     const int u = blockIdx.x * blockDim.x + threadIdx.x;
     const bool in = u < U;
     const int c = in ? preSum[u + 1] - preSum[u] : 0;
     const int wmax = wave_max_i32(c);
-    const int n_empty = __popcll(__ballot(in && c == 0));
     const bool mismatch = in && unq_cnts && unq_cnts[u] != (long long)c;
     const int any_mismatch = __ballot(mismatch) != 0ull;
     const int w = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) {
         s_max[w] = wmax;
-        s_empty[w] = n_empty;
         s_bad[w] = any_mismatch;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        int m = 0, e = 0, b = 0;
+        int m = 0, b = 0;
         for (int k = 0; k < kSpecialThreads / 64; ++k) {
             m = max(m, s_max[k]);
-            e += s_empty[k];
             b |= s_bad[k];
         }
         if (m > 0) atomicMax(&stats[TXS_STAT_MAX_CNT], m);
-        if (e) atomicAdd(&stats[TXS_STAT_NUM_EMPTY], e);
         if (b) stats[TXS_STAT_COUNT_MISMATCH] = 1;
     }
+    if (in && cnts_out) cnts_out[u] = (long long)c;
+    // Slots: heavy voxels fill heavy_ids from the front (their slot is also their row in
+    // the scratch table), empty voxels from the back of the U-entry array (they own no
+    // scratch).  One atomic per wave and kind hands out a contiguous range.
+    const bool heavy = in && c > heavy_threshold;
+    const bool empty = in && c == 0;
+    const unsigned long long mh = __ballot(heavy), me = __ballot(empty);
+    const int lane = threadIdx.x & 63;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    int base_h = 0, base_e = 0;
+    if (lane == 0) {
+        if (mh) base_h = atomicAdd(&stats[TXS_STAT_NUM_HEAVY], __popcll(mh));
+        if (me) base_e = atomicAdd(&stats[TXS_STAT_NUM_EMPTY], __popcll(me));
+        if (mh | me) atomicAdd(&stats[TXS_STAT_NUM_SPECIAL], __popcll(mh) + __popcll(me));
+    }
+    base_h = __shfl(base_h, 0, 64);
+    base_e = __shfl(base_e, 0, 64);
     if (!in) return;
-    if (cnts_out) cnts_out[u] = (long long)c;
     int slot = -1;
-    if (c > heavy_threshold || c == 0) {
-        slot = atomicAdd(&stats[TXS_STAT_NUM_SPECIAL], 1);
-        if (slot < U) heavy_ids[slot] = u;
+    if (heavy) {
+        slot = base_h + __popcll(mh & below);
+        if (slot < U_arg) heavy_ids[slot] = u;
+    } else if (empty) {
+        slot = U_arg - 1 - (base_e + __popcll(me & below));
+        if (slot >= 0) heavy_ids[slot] = u;
     }
     slot_of[u] = slot;
 }

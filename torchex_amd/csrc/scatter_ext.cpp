@@ -71,6 +71,15 @@ std::vector<int64_t> read_stats(const Tensor &stats) {
     return v;
 }
 
+// The special-voxel list the forward call takes: txs_plan_special leaves the heavy
+// voxels at the front of its `capacity`-entry array and the empty ones at its back.
+Tensor special_list(const Tensor &heavy_all, int64_t capacity, const std::vector<int64_t> &hs) {
+    const int64_t n_heavy = hs[TXS_STAT_NUM_HEAVY], n_empty = hs[TXS_STAT_NUM_EMPTY];
+    Tensor heavy = heavy_all.narrow(0, 0, n_heavy);
+    if (n_empty == 0) return heavy.contiguous();
+    return at::cat({heavy, heavy_all.narrow(0, capacity - n_empty, n_empty)});
+}
+
 // ScatterData index preparation for an unq_inv in any order
 // (extends torchex/operator_py/scatter_op.py:13-21).  Everything is queued on
 // the current stream; the only host synchronisation is the read of `stats`.
@@ -111,7 +120,7 @@ std::tuple<Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>> buil
                 "unq_inv holds ids outside [0, num_unq=", U, ")");
     OptTensor perm_out;
     if (hs[TXS_STAT_UNSORTED]) perm_out = perm;
-    Tensor heavy_ids = heavy_all.narrow(0, 0, hs[TXS_STAT_NUM_SPECIAL]).contiguous();
+    Tensor heavy_ids = special_list(heavy_all, U, hs);
     return {preSum, perm_out, seg, slot_of, heavy_ids, hs};
 }
 
@@ -135,7 +144,7 @@ std::tuple<Tensor, Tensor, Tensor, std::vector<int64_t>> plan_from_presum(
         check_status(txs_plan_seg_from_presum(i32p(preSum), N, U, i32p(slot_of), i32w(seg), st),
                      "plan_seg_from_presum");
     std::vector<int64_t> hs = read_stats(stats);
-    Tensor heavy_ids = heavy_all.narrow(0, 0, hs[TXS_STAT_NUM_SPECIAL]).contiguous();
+    Tensor heavy_ids = special_list(heavy_all, U, hs);
     return {seg, slot_of, heavy_ids, hs};
 }
 
@@ -205,7 +214,7 @@ unique_plan(const Tensor &keys, int64_t key_bound, int64_t heavy_threshold, cons
     OptTensor perm_out;
     if (hs[TXS_STAT_UNSORTED]) perm_out = perm;
     return {unq.narrow(0, 0, U), inv, cnts.narrow(0, 0, U), preSum.narrow(0, 0, U + 1), perm_out, seg,
-            slot_of.narrow(0, 0, U), heavy_all.narrow(0, 0, hs[TXS_STAT_NUM_SPECIAL]).contiguous(), hs};
+            slot_of.narrow(0, 0, U), special_list(heavy_all, N, hs), hs};
 }
 
 // ingroup_inds(seg, perm | None, preSum, num_unq) -> int64 [N]
@@ -292,8 +301,9 @@ Tensor grid_hash_probe(const Tensor &coors, const Tensor &table) {
     return out;
 }
 
-Tensor make_scratch(int64_t num_special, int64_t C, const Tensor &like) {
-    return at::zeros({num_special * C}, like.options().dtype(at::kLong));
+// one zeroed row of 8-byte cells per heavy voxel (empty voxels need none)
+Tensor make_scratch(int64_t num_heavy, int64_t C, const Tensor &like) {
+    return at::zeros({num_heavy, C}, like.options().dtype(at::kLong));
 }
 
 void run_forward(int op, const Tensor &feats, const OptTensor &perm, const Tensor &seg,
@@ -301,11 +311,14 @@ void run_forward(int op, const Tensor &feats, const OptTensor &perm, const Tenso
                  Tensor &scratch, Tensor &out, OptTensor &arg, int64_t max_cnt) {
     const int64_t N = feats.size(0), C = feats.size(1), U = preSum.numel() - 1;
     const int64_t S = heavy_ids.numel();
+    TORCH_CHECK(scratch.dim() == 2 && (scratch.size(0) == 0 || scratch.size(1) == C),
+                "scratch must be [num_heavy, channel] (ScatterData.scratch(channel))");
+    const int64_t H = scratch.size(0);
+    TORCH_CHECK(H <= S, "scratch has more rows than there are special voxels");
     TORCH_CHECK(seg.numel() == N, "plan was built for ", seg.numel(), " rows, feats has ", N);
     TORCH_CHECK(!perm.has_value() || perm->numel() == N, "perm length mismatch");
     TORCH_CHECK(slot_of.numel() == U, "slot_of length mismatch");
     TORCH_CHECK(out.size(0) == U && out.size(1) == C, "out must be [num_unq, channel]");
-    TORCH_CHECK(S == 0 || scratch.numel() >= S * C, "scratch too small");
     const int dt = dtype_code(feats, "feats");
     void *st = cur_stream(feats);
     int rc;
@@ -313,7 +326,7 @@ void run_forward(int op, const Tensor &feats, const OptTensor &perm, const Tenso
         pybind11::gil_scoped_release nogil;
         rc = txs_scatter_forward(op, dt, feats.data_ptr(), opt_i32p(perm), i32p(seg), i32p(preSum),
                                  i32p(slot_of), i32p(heavy_ids), S,
-                                 S ? scratch.data_ptr() : nullptr, out.data_ptr(),
+                                 H ? scratch.data_ptr() : nullptr, out.data_ptr(),
                                  arg.has_value() ? arg->data_ptr<int32_t>() : nullptr, N, C, U, max_cnt,
                                  st);
     }
@@ -388,7 +401,7 @@ void csr_reduce(int op, Tensor feats, Tensor preSum, Tensor out, OptTensor arg, 
     c10::hip::HIPGuardMasqueradingAsCUDA guard(feats.device());
     auto [seg, slot_of, heavy_ids, hs] =
         plan_from_presum(preSum, feats.size(0), txs_default_heavy_threshold());
-    Tensor scratch = make_scratch(heavy_ids.numel(), feats.size(1), feats);
+    Tensor scratch = make_scratch(hs[TXS_STAT_NUM_HEAVY], feats.size(1), feats);
     OptTensor perm;
     run_forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, out, arg, max_cnt);
 }

@@ -420,6 +420,15 @@ __global__ void scatter_finalize_kernel(const typename TR::raw *__restrict__ fea
     const int u = heavy_ids[s];
     if ((unsigned)u >= (unsigned)U) return;
     const size_t o = (size_t)u * C + c;
+    if (preSum[u + 1] == preSum[u]) {  // empty voxel: listed after the heavy ones, owns no scratch row
+        if (OP == TXS_MAX || OP == TXS_MAX_REFTIE) {
+            out[o] = TR::lowest();
+            arg[o] = -1;
+        } else {
+            out[o] = TR::from_f(OP == TXS_MEAN ? __builtin_nanf("") : 0.0f);  // mean: 0/0 as in the reference
+        }
+        return;
+    }
     if (OP == TXS_MAX || OP == TXS_MAX_REFTIE) {
         const unsigned long long key = scratch[t];
         scratch[t] = 0ull;
@@ -746,7 +755,7 @@ hipError_t launch_bwd(int op, const Geometry &geo, hipStream_t st, const void *g
 
 extern "C" {
 
-int txs_abi_version(void) { return 5; }
+int txs_abi_version(void) { return 6; }
 
 const char *txs_status_string(int status) {
     switch (status) {
@@ -779,7 +788,7 @@ int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *per
     int ref_log2 = 5;
     while (ref_log2 < 10 && (1LL << ref_log2) < max_cnt) ++ref_log2;
     if (num_total > 0 && (!feats || !seg || !slot_of)) return TXS_ERR_INVALID_ARG;
-    if (num_special > 0 && (!scratch || !heavy_ids)) return TXS_ERR_INVALID_ARG;
+    if (num_special > 0 && !heavy_ids) return TXS_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const int N = (int)num_total, C = (int)channel, U = (int)num_unq;
     const int elem = dtype == TXS_F32 ? 4 : 2;

@@ -65,6 +65,7 @@ class ScatterData:
         self.is_sorted = self.perm is None
         self.max_cnt = int(stats[2])
         self.num_special = int(stats[3])
+        self.num_heavy = int(stats[7])
         self.num_unq = num_unq
         self._scratch = {}
 
@@ -93,6 +94,7 @@ class ScatterData:
         self.is_sorted = self.perm is None
         self.max_cnt = int(stats[2])
         self.num_special = int(stats[3])
+        self.num_heavy = int(stats[7])
         self.num_unq = int(stats[6])
         self._scratch = {}
         return self
@@ -111,14 +113,14 @@ class ScatterData:
         return self
 
     def scratch(self, channel):
-        """Zeroed table the special voxels are merged in; the kernels leave it
+        """Zeroed table the heavy voxels are merged in (one row each); the kernels leave it
         zeroed again, so one buffer per channel count is kept for reuse.  Forward
         calls that share a ``ScatterData`` therefore must not overlap in time on the
         GPU (two streams running them concurrently would race on this table); calls
         on one stream, the normal case, are ordered."""
         buf = self._scratch.get(channel)
         if buf is None:
-            buf = scatter_ext.make_scratch(self.num_special, channel, self.seg)
+            buf = scatter_ext.make_scratch(self.num_heavy, channel, self.seg)
             self._scratch[channel] = buf
         return buf
 
