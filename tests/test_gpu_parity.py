@@ -763,3 +763,40 @@ def test_mostly_empty_voxel_grid():
     # layout the kernels rely on: heavy voxels first, then the empty ones
     ids = data.heavy_ids.cpu()
     assert ids[0].item() == 123_456 and bool((cnts[ids[1:].long()] == 0).all())
+
+
+def test_reference_style_module_calls_reuse_their_plan():
+    """scatter_ext.sum / max take only CSR offsets (the reference's signatures).  The
+    plan behind a preSum tensor is kept between calls; it is rebuilt when the tensor is
+    rewritten in place or used with another row count."""
+    import scatter_ext
+    scatter_ext.clear_csr_plan_cache()
+    sizes = torch.tensor([3, 1, 70, 2, 5, 130, 1, 1, 9], dtype=torch.long)
+    U, N, C = sizes.numel(), int(sizes.sum()), 12
+    inv = torch.repeat_interleave(torch.arange(U), sizes)
+    g = torch.Generator().manual_seed(8)
+    feats = torch.randn((N, C), generator=g)
+    pre = torch.zeros(U + 1, dtype=torch.int32, device=DEV)
+    scatter_ext.getPreSum(inv.int().to(DEV), pre)
+    f = feats.to(DEV)
+    want = orc.scatter_sum_f64(feats.numpy(), inv.numpy().astype(np.int32), U)
+    wm, wa = orc.scatter_max_reforder(feats.numpy(), inv.numpy().astype(np.int32), U)
+    for _ in range(3):                                   # first call builds, the others reuse
+        out = torch.zeros((U, C), device=DEV)
+        scatter_ext.sum(f, pre, out, int(sizes.max()))
+        assert np.allclose(out.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+        mx = torch.zeros((U, C), device=DEV)
+        arg = torch.zeros((U, C), device=DEV, dtype=torch.int32)
+        scatter_ext.max(f, pre, mx, arg, int(sizes.max()))
+        assert np.array_equal(arg.cpu().numpy(), wa) and bits_equal(mx.cpu().numpy(), wm)
+    # the same tensor rewritten in place for other voxel sizes: the old plan must not be used
+    sizes2 = torch.tensor([100, 1, 1, 2, 5, 10, 1, 1, 100], dtype=torch.long)
+    assert int(sizes2.sum()) == N - 1
+    inv2 = torch.repeat_interleave(torch.arange(U), sizes2)
+    scatter_ext.getPreSum(inv2.int().to(DEV), pre)
+    f2 = f[:N - 1].contiguous()
+    out = torch.zeros((U, C), device=DEV)
+    scatter_ext.sum(f2, pre, out, 100)
+    want2 = orc.scatter_sum_f64(feats[:N - 1].numpy(), inv2.numpy().astype(np.int32), U)
+    assert np.allclose(out.cpu().numpy(), want2, rtol=1e-5, atol=1e-5)
+    scatter_ext.clear_csr_plan_cache()

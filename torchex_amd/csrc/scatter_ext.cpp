@@ -16,8 +16,10 @@
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
+#include <algorithm>
 #include <optional>
 #include <tuple>
+#include <utility>
 #include <vector>
 
 #include "torchex_scatter.h"
@@ -391,6 +393,50 @@ Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const 
 
 // ---- the reference module's three functions (scatter.cpp:20-64) ------------
 
+// The reference module's entry points take only CSR offsets, every call.  The plan that
+// goes with a preSum tensor is kept for the next calls (the reference's ScatterData
+// makes preSum once and then calls sum/max many times): a few entries, keyed by the
+// tensor's storage, length and version, each holding the tensor itself so that its
+// storage cannot be handed to another tensor while the entry lives.
+struct CsrPlan {
+    Tensor preSum, seg, slot_of, heavy_ids;
+    uint32_t version = 0;
+    int64_t num_total = 0, num_heavy = 0;
+    std::vector<std::pair<int64_t, Tensor>> scratch;  // per channel count
+};
+constexpr size_t kCsrPlanCacheSize = 8;
+std::vector<CsrPlan> &csr_plan_cache() {
+    // touched under the GIL only; never destroyed, so no device tensor is freed after
+    // the runtime has shut down at interpreter exit
+    static auto *cache = new std::vector<CsrPlan>();
+    return *cache;
+}
+
+CsrPlan &csr_plan_for(const Tensor &preSum, int64_t num_total) {
+    auto &cache = csr_plan_cache();
+    const uint32_t version = preSum.unsafeGetTensorImpl()->version_counter().current_version();
+    for (size_t i = 0; i < cache.size(); ++i) {
+        CsrPlan &p = cache[i];
+        if (p.preSum.data_ptr() == preSum.data_ptr() && p.preSum.numel() == preSum.numel() &&
+            p.preSum.device() == preSum.device() && p.version == version && p.num_total == num_total) {
+            if (i != 0) std::rotate(cache.begin(), cache.begin() + i, cache.begin() + i + 1);  // most recent first
+            return cache.front();
+        }
+    }
+    auto [seg, slot_of, heavy_ids, hs] = plan_from_presum(preSum, num_total, txs_default_heavy_threshold());
+    CsrPlan p;
+    p.preSum = preSum;
+    p.seg = seg;
+    p.slot_of = slot_of;
+    p.heavy_ids = heavy_ids;
+    p.version = version;
+    p.num_total = num_total;
+    p.num_heavy = hs[TXS_STAT_NUM_HEAVY];
+    if (cache.size() >= kCsrPlanCacheSize) cache.pop_back();
+    cache.insert(cache.begin(), std::move(p));
+    return cache.front();
+}
+
 void csr_reduce(int op, Tensor feats, Tensor preSum, Tensor out, OptTensor arg, int64_t max_cnt) {
     check_dev(feats, "feats");
     check_i32(preSum, "preSum");
@@ -399,12 +445,20 @@ void csr_reduce(int op, Tensor feats, Tensor preSum, Tensor out, OptTensor arg, 
     TORCH_CHECK(out.scalar_type() == feats.scalar_type(), "out dtype must match feats");
     TORCH_CHECK(preSum.numel() == out.size(0) + 1, "preSum must have out.size(0)+1 entries");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(feats.device());
-    auto [seg, slot_of, heavy_ids, hs] =
-        plan_from_presum(preSum, feats.size(0), txs_default_heavy_threshold());
-    Tensor scratch = make_scratch(hs[TXS_STAT_NUM_HEAVY], feats.size(1), feats);
+    CsrPlan &plan = csr_plan_for(preSum, feats.size(0));
+    const int64_t C = feats.size(1);
+    Tensor scratch;
+    for (auto &kv : plan.scratch)
+        if (kv.first == C) scratch = kv.second;
+    if (!scratch.defined()) {
+        scratch = make_scratch(plan.num_heavy, C, feats);
+        plan.scratch.emplace_back(C, scratch);
+    }
     OptTensor perm;
-    run_forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, out, arg, max_cnt);
+    run_forward(op, feats, perm, plan.seg, preSum, plan.slot_of, plan.heavy_ids, scratch, out, arg, max_cnt);
 }
+
+void clear_csr_plan_cache() { csr_plan_cache().clear(); }
 
 // sum(feats, preSum, out, max_cnt): max_cnt only shaped the reference's thread
 // blocks (scatter_kernel.cu:179); it does not change a sum and is not needed here.
@@ -444,7 +498,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("dynamic_point_pool", &dynamic_point_pool, "dynamic_point_pool(rois, pts, extra_wlh, max_pts_per_box, max_all_pts)");
     m.def("grid_hash_build", &grid_hash_build, "build_table(coors, values) -> table");
     m.def("grid_hash_probe", &grid_hash_probe, "probe_table(coors, table) -> values");
-    m.def("make_scratch", &make_scratch, "zeroed scratch table for the special voxels");
+    m.def("make_scratch", &make_scratch, "zeroed scratch table, one row per heavy voxel");
+    m.def("clear_csr_plan_cache", &clear_csr_plan_cache, "drop the plans kept for sum/max over CSR offsets");
     m.def("forward", &forward, "forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, max_cnt)");
     m.def("backward", &backward, "backward(op, grad_out, arg, perm, seg, preSum, num_total)");
     m.def("abi_version", &txs_abi_version);
