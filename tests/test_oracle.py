@@ -464,3 +464,45 @@ def test_grid_hash_oracle():
     keys2 = rng.choice(10 ** 6, size=1024, replace=False).astype(np.int32)
     t2 = orc.grid_hash_build(keys2, np.arange(1024, dtype=np.int32))
     assert (t2[:, 0] != -1).all() and np.array_equal(orc.grid_hash_probe(keys2, t2), np.arange(1024))
+
+
+def test_property_random_small_inputs_against_python_loops():
+    """Hypothesis-driven: the C oracle's spec functions against plain Python loops on
+    small random inputs with planted ties, signed zeros and empty voxels."""
+    from hypothesis import given, settings, strategies as st
+
+    vals = st.sampled_from([-2.0, -1.0, -0.0, 0.0, 0.5, 1.0, 1.0, 3.0])
+
+    @settings(max_examples=80, deadline=None)
+    @given(st.integers(1, 6).flatmap(lambda U: st.tuples(
+        st.just(U), st.lists(st.tuples(st.integers(0, U - 1), vals, vals), min_size=1, max_size=40))))
+    def check(case):
+        U, rows = case
+        inv = np.array([r[0] for r in rows], dtype=np.int32)
+        f = np.array([[r[1], r[2]] for r in rows], dtype=np.float32)
+        N, C = f.shape
+        s = orc.scatter_sum_f64(f, inv, U)
+        mx, arg = orc.scatter_max_first(f, inv, U)
+        cnt = orc.counts(inv, U)
+        for u in range(U):
+            members = [i for i in range(N) if inv[i] == u]
+            assert cnt[u] == len(members)
+            for c in range(C):
+                assert s[u, c] == sum(float(f[i, c]) for i in members)
+                if not members:
+                    assert arg[u, c] == -1
+                    continue
+                best = members[0]
+                for i in members[1:]:
+                    if f[i, c] > f[best, c]:      # strict: the first of equal maxima stays
+                        best = i
+                assert arg[u, c] == best
+                assert mx[u, c].tobytes() == f[best, c].tobytes()
+        g = np.arange(U * C, dtype=np.float32).reshape(U, C) + 1
+        gin = orc.max_backward(g, arg, N)
+        for i in range(N):
+            for c in range(C):
+                assert gin[i, c] == (g[inv[i], c] if arg[inv[i], c] == i else 0.0)
+        assert np.array_equal(orc.sum_backward(g, inv), g[inv])
+
+    check()
