@@ -171,6 +171,8 @@ def frontend_timings(T, workloads, dev, N):
     frontend["voxelize_ms"] = wall_ms(lambda: T.voxelize(pts, [0.2, 0.2, 0.2], [-75, -75, -2, 75, 75, 4]), 20)
     frontend["torch_div_floor_voxelize_ms"] = wall_ms(
         lambda: torch.div(pts[:, :3] - lo_t[None, :], vs_t[None, :], rounding_mode="floor").int(), 20)
+    i2 = torch.unique(keys, return_inverse=True)[1]
+    frontend["ingroup_inds_ms"] = wall_ms(lambda: T.ingroup_inds(i2))
     frontend["ScatterData_from_points_ms"] = wall_ms(
         lambda: T.ScatterData.from_points(pts, [0.2, 0.2, 0.2], [-75, -75, -2, 75, 75, 4]))
 
