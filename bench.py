@@ -315,7 +315,8 @@ def main():
 
     dom = max(("max_fwd", "max_bwd", "mean_fwd", "mean_bwd"), key=lambda k: kt[k])
     row_bytes = C * esz
-    vec = next(v for v in (16, 8, 4, 2) if row_bytes % v == 0 and v >= esz) // esz   # elements per lane
+    # elements per lane: 16-byte vectors for fp32, 8-byte ones for the 2-byte types
+    vec = next(v for v in ((16, 8, 4) if esz == 4 else (8, 4, 2)) if row_bytes % v == 0) // esz
     kname = "scatter_%s_kernel<%s,%d,%s>" % (dom[-3:], a.dtype.upper(), vec, dom[:-4].upper())
     if dom.endswith("bwd"):   # the backward kernel also carries its chunk (positions per lane group)
         kname = kname[:-1] + (",8>" if N < 16 * U else ",16>")

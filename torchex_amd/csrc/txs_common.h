@@ -41,6 +41,7 @@ constexpr int kChunkBwdShort = TXS_CHUNK_BWD_SHORT;  // backward kernel, mean ru
 constexpr int kChunkBwdLong = TXS_CHUNK;             // backward kernel, longer runs
 constexpr int kBatchBwd = TXS_BATCH_BWD;
 constexpr int kBatch = TXS_BATCH;    // rows per load batch of a lane group (two batches in flight)
+constexpr int kHalfVecBytes = 8;     // bytes one lane moves per row for fp16 / bf16
 constexpr int kHeavyDefault = 64;    // voxels above this many rows use the atomic path
 constexpr int kSpecialBit = (int)0x80000000;
 constexpr int kIdMask = 0x7fffffff;
