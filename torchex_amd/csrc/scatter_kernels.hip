@@ -278,17 +278,16 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
 
     // Every slot of a batch issues a load (slots past the range re-load the
     // range's last row, a cache hit) so that no load sits under a branch.
+    // A batch keeps only the loaded rows; the voxel and row ids are read again from LDS
+    // when the batch is reduced (fewer live registers: one more wave per SIMD for sum/mean).
     struct Batch {
-        int segs[kBatch], rows[kBatch];
         Pack<raw, VEC> v[kBatch];
     };
     auto issue = [&](Batch &bt, int l) {
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
             const int lc = min(l + i, lb_fast - 1);
-            bt.segs[i] = seg_s[lc];
-            bt.rows[i] = perm_s[lc - 1];
-            bt.v[i] = ld_stream<raw, VEC>(row_ptr(bt.rows[i]));
+            bt.v[i] = ld_stream<raw, VEC>(row_ptr(perm_s[lc - 1]));
         }
     };
     // A batch that lies wholly inside the range needs no per-row gate; only the
@@ -296,12 +295,14 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     auto consume_full = [&](const Batch &bt, int l) {
 #pragma unroll
         for (int i = 0; i < kBatch; ++i)
-            add_row(std::false_type{}, bt.v[i], bt.segs[i], bt.rows[i], l + i, true);
+            add_row(std::false_type{}, bt.v[i], seg_s[l + i], perm_s[l + i - 1], l + i, true);
     };
     auto consume_last = [&](const Batch &bt, int l) {
 #pragma unroll
-        for (int i = 0; i < kBatch; ++i)
-            add_row(std::true_type{}, bt.v[i], bt.segs[i], bt.rows[i], l + i, l + i < lb_fast);
+        for (int i = 0; i < kBatch; ++i) {
+            const int lc = min(l + i, lb_fast - 1);
+            add_row(std::true_type{}, bt.v[i], seg_s[lc], perm_s[lc - 1], l + i, l + i < lb_fast);
+        }
     };
 
     // Positions staged in LDS go through the double-buffered loop; the rare rest
