@@ -63,7 +63,7 @@ enum {
     TXS_STATS_LEN = 8
 };
 
-/* Library ABI version; bumped when a signature changes. */
+/* Library ABI version (6); bumped when a signature or the meaning of an argument changes. */
 int txs_abi_version(void);
 
 /* Human-readable text for a status code. */
