@@ -800,3 +800,25 @@ def test_reference_style_module_calls_reuse_their_plan():
     want2 = orc.scatter_sum_f64(feats[:N - 1].numpy(), inv2.numpy().astype(np.int32), U)
     assert np.allclose(out.cpu().numpy(), want2, rtol=1e-5, atol=1e-5)
     scatter_ext.clear_csr_plan_cache()
+
+
+def test_assume_sorted_skips_the_sort_and_is_verified():
+    """ScatterData(..., assume_sorted=True) on grouped input (the reference's contract)
+    builds the same plan without queueing the sort; an input that is not sorted raises."""
+    T = tx()
+    w = workloads.lidar_sweep(N=100_000, C=32, seed=41)
+    order = torch.sort(w.unq_inv, stable=True)[1]
+    inv_s, f_s = w.unq_inv[order].to(DEV), w.feats[order].to(DEV)
+    cnts = w.unq_cnts.to(DEV)
+    a = T.ScatterData(inv_s, cnts)
+    b = T.ScatterData(inv_s, cnts, assume_sorted=True)
+    assert a.is_sorted and b.is_sorted and b.perm is None
+    for name in ("preSum", "seg", "slot_of", "heavy_ids"):
+        assert torch.equal(getattr(a, name), getattr(b, name)), name
+    assert (a.max_cnt, a.num_special, a.num_heavy) == (b.max_cnt, b.num_special, b.num_heavy)
+    ma, aa = T.scatter_max(f_s, a)
+    mb, ab = T.scatter_max(f_s, b)
+    assert torch.equal(ma, mb) and torch.equal(aa, ab)
+    assert torch.equal(T.scatter_mean(f_s, a), T.scatter_mean(f_s, b))
+    with pytest.raises(RuntimeError, match="declared sorted"):
+        T.ScatterData(w.unq_inv.to(DEV), cnts, assume_sorted=True)

@@ -86,8 +86,12 @@ Tensor special_list(const Tensor &heavy_all, int64_t capacity, const std::vector
 // (extends torchex/operator_py/scatter_op.py:13-21).  Everything is queued on
 // the current stream; the only host synchronisation is the read of `stats`.
 // returns (preSum, perm | None, seg, slot_of, heavy_ids, stats)
+// assume_sorted: the caller states that unq_inv is non-decreasing (the only order the
+// reference accepts); the sort is then not even queued, and the statement is checked
+// on the device (an unsorted unq_inv raises).
 std::tuple<Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>> build_plan(
-    const Tensor &unq_inv, int64_t num_unq, int64_t heavy_threshold, const OptTensor &unq_cnts) {
+    const Tensor &unq_inv, int64_t num_unq, int64_t heavy_threshold, const OptTensor &unq_cnts,
+    bool assume_sorted) {
     check_i32(unq_inv, "unq_inv");
     TORCH_CHECK(unq_inv.dim() == 1, "unq_inv must be 1-D");
     TORCH_CHECK(num_unq >= 0, "num_unq must be non-negative");
@@ -102,16 +106,21 @@ std::tuple<Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>> buil
     const int64_t N = unq_inv.numel(), U = num_unq;
     void *st = cur_stream(unq_inv);
     Tensor stats = at::zeros({TXS_STATS_LEN}, unq_inv.options());
-    Tensor seg = empty_i32(N, unq_inv);
-    Tensor perm = empty_i32(N, unq_inv);
-    Tensor ws = empty_i32(txs_sort_workspace_len(N, U), unq_inv);
+    Tensor seg, perm;
     Tensor preSum = empty_i32(U + 1, unq_inv);
     Tensor slot_of = empty_i32(U, unq_inv);
     Tensor heavy_all = empty_i32(U, unq_inv);
     check_status(txs_plan_check(i32p(unq_inv), N, U, i32w(stats), st), "plan_check");
-    if (U > 0)
-        check_status(txs_plan_sort(i32p(unq_inv), N, U, i32p(stats), i32w(perm), i32w(seg), i32w(ws), st),
-                     "plan_sort");
+    if (assume_sorted) {
+        seg = unq_inv.clone();  // sorted ids are their own sorted keys
+    } else {
+        seg = empty_i32(N, unq_inv);
+        perm = empty_i32(N, unq_inv);
+        Tensor ws = empty_i32(txs_sort_workspace_len(N, U), unq_inv);
+        if (U > 0)
+            check_status(txs_plan_sort(i32p(unq_inv), N, U, i32p(stats), i32w(perm), i32w(seg), i32w(ws), st),
+                         "plan_sort");
+    }
     check_status(txs_plan_presum(i32p(seg), U > 0 ? N : 0, U, i32w(preSum), st), "plan_presum");
     check_status(txs_plan_special(i32p(preSum), U, (int32_t)heavy_threshold, cnts, i32w(slot_of),
                                   i32w(heavy_all), i32w(stats), nullptr, nullptr, st),
@@ -120,6 +129,8 @@ std::tuple<Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>> buil
     std::vector<int64_t> hs = read_stats(stats);
     TORCH_CHECK(hs[TXS_STAT_OUT_OF_RANGE] == 0 && (U > 0 || N == 0),
                 "unq_inv holds ids outside [0, num_unq=", U, ")");
+    TORCH_CHECK(!(assume_sorted && hs[TXS_STAT_UNSORTED]),
+                "unq_inv was declared sorted (assume_sorted=True) but is not non-decreasing");
     OptTensor perm_out;
     if (hs[TXS_STAT_UNSORTED]) perm_out = perm;
     Tensor heavy_ids = special_list(heavy_all, U, hs);
@@ -490,7 +501,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("sum", &sum_ref, "scatter_sum over CSR offsets, in place (HIP)");
     m.def("max", &max_ref, "scatter_max with arg over CSR offsets, in place (HIP)");
     m.def("getPreSum", &get_presum_ref, "CSR offsets from a sorted unq_inv (HIP)");
-    m.def("build_plan", &build_plan, "build_plan(unq_inv, num_unq, heavy_threshold, unq_cnts|None)");
+    m.def("build_plan", &build_plan, "build_plan(unq_inv, num_unq, heavy_threshold, unq_cnts|None, assume_sorted=False)",
+          pybind11::arg("unq_inv"), pybind11::arg("num_unq"), pybind11::arg("heavy_threshold"),
+          pybind11::arg("unq_cnts"), pybind11::arg("assume_sorted") = false);
     m.def("plan_from_presum", &plan_from_presum, "index preparation from CSR offsets");
     m.def("voxel_keys", &voxel_keys, "voxel_keys(points, range_lo, voxel_size, dims) -> (coors, keys, stats)");
     m.def("unique_plan", &unique_plan, "unique_plan(keys, key_bound, heavy_threshold, stats|None)");

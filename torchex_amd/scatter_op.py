@@ -33,9 +33,14 @@ class ScatterData:
     ``None`` when ``unq_inv`` is already non-decreasing), ``seg`` (int32 ``[N]``
     voxel at each sorted position, bit 31 marking voxels reduced through
     atomics), ``slot_of`` / ``heavy_ids`` (table of those voxels).
+
+    ``assume_sorted=True`` states that ``unq_inv`` is already grouped (the order the
+    reference requires): the sort is then not queued at all; the statement is
+    verified on the device and an unsorted ``unq_inv`` raises.
     """
 
-    def __init__(self, unq_inv, unq_cnts, heavy_threshold=None, max_tie_rule="first") -> None:
+    def __init__(self, unq_inv, unq_cnts, heavy_threshold=None, max_tie_rule="first",
+                 assume_sorted=False) -> None:
         assert unq_inv.ndim in (
             1, 2), f"unq_inv in ScatterData should be 1 or 2-dims, but got {unq_inv.ndim}-dims"
         assert unq_cnts.ndim in (
@@ -57,7 +62,7 @@ class ScatterData:
         num_unq = self.unq_cnts.shape[0]
         cnts64 = self.unq_cnts.reshape(-1).long().contiguous()
         (self.preSum, self.perm, self.seg, self.slot_of, self.heavy_ids,
-         stats) = scatter_ext.build_plan(flat, num_unq, self.heavy_threshold, cnts64)
+         stats) = scatter_ext.build_plan(flat, num_unq, self.heavy_threshold, cnts64, bool(assume_sorted))
         # same consistency check as the reference (scatter_op.py:19), made on
         # the recomputed histogram so that a stale unq_cnts is caught too
         assert stats[5] == 0, "unq_cnts is not the histogram of unq_inv"
