@@ -41,7 +41,8 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
-_SPECIAL = {"NZ": -0.0, "NI": -np.inf, "PI": np.inf, "NAN": np.nan}
+_SPECIAL = {"NZ": -0.0, "NI": -np.inf, "PI": np.inf, "NAN": np.nan,
+            "NFLTMAX": -float(np.finfo(np.float32).max)}
 
 
 def _decode(x):
@@ -61,7 +62,7 @@ def load_hand_cases():
         for k, v in c.items():
             if k in ("name", "inv"):
                 continue
-            dt = np.int32 if k == "arg" else np.float32
+            dt = np.int32 if k in ("arg", "arg_ref") else np.float32
             d[k] = np.array(_decode(v), dtype=dt)
         cases.append(d)
     return cases

@@ -244,6 +244,12 @@ def test_dynamic_point_pool_feeds_the_scatter_path():
     assert data.is_sorted                               # (box, point) order: no permutation needed
     mx, arg = T.scatter_max(feats.contiguous(), data)
     unq, inv = torch.unique(roi.cpu(), return_inverse=True)
+    # grouped rows: the default reports the reference kernel's winner among equal maxima
+    assert data.max_tie_rule == "reference"
+    wm, wa = orc.scatter_max_reforder(feats.cpu().numpy(), inv.numpy().astype(np.int32), unq.shape[0])
+    assert np.array_equal(arg.cpu().numpy(), wa) and np.array_equal(mx.cpu().numpy(), wm)
+    d1 = T.ScatterData.from_keys(roi, 50, max_tie_rule="first")
+    mx, arg = T.scatter_max(feats.contiguous(), d1)
     wm, wa = orc.scatter_max_first(feats.cpu().numpy(), inv.numpy().astype(np.int32), unq.shape[0])
     assert np.array_equal(arg.cpu().numpy(), wa) and np.array_equal(mx.cpu().numpy(), wm)
 

@@ -44,9 +44,11 @@ def bits_equal(a, b):
 
 
 def run_case(name, feats, unq_inv, unq_cnts, dtype=torch.float32, grad_seed=100, check_plan=True,
-             heavy_threshold=None):
+             heavy_threshold=None, max_tie_rule=None):
     """feats fp32 CPU [N, C]; unq_inv int64 CPU; unq_cnts int64 CPU.  Returns the
-    ScatterData for extra checks."""
+    ScatterData for extra checks.  scatter_max is checked against the oracle of the tie
+    rule in force: by default the reference kernel's own winner (lane-exact emulation)
+    when the rows are grouped by voxel, the smallest row otherwise."""
     T = tx()
     N, C = feats.shape
     U = unq_cnts.shape[0]
@@ -57,7 +59,11 @@ def run_case(name, feats, unq_inv, unq_cnts, dtype=torch.float32, grad_seed=100,
     cnt = unq_cnts.numpy()
 
     fg = f_in.to(DEV).requires_grad_(True)
-    data = T.ScatterData(unq_inv.to(DEV), unq_cnts.to(DEV), heavy_threshold=heavy_threshold)
+    data = T.ScatterData(unq_inv.to(DEV), unq_cnts.to(DEV), heavy_threshold=heavy_threshold,
+                         max_tie_rule=max_tie_rule)
+    grouped = N < 2 or bool((unq_inv[1:] >= unq_inv[:-1]).all())
+    assert data.is_sorted == grouped
+    assert data.max_tie_rule == (max_tie_rule or ("reference" if grouped else "first"))
 
     # ---- index preparation: integers, exact
     want_pre = orc.presum(orc.counts(inv32, U))
@@ -95,7 +101,10 @@ def run_case(name, feats, unq_inv, unq_cnts, dtype=torch.float32, grad_seed=100,
                   (rt * sabs[nz] / cnt[nz, None] + oe * np.abs(wantm))[fm] + 1e-30), "mean"
     assert np.all(np.isnan(gotm[~nz])), "mean of an empty voxel is 0/0 as in the reference"
 
-    want_max, want_arg = orc.scatter_max_first(f32, inv32, U)
+    if data.max_tie_rule == "reference":
+        want_max, want_arg = orc.scatter_max_reforder(f32, inv32, U)
+    else:
+        want_max, want_arg = orc.scatter_max_first(f32, inv32, U)
     got_arg = arg.cpu().numpy()
     assert np.array_equal(got_arg, want_arg), \
         f"arg: {int((got_arg != want_arg).sum())} of {want_arg.size} differ"
@@ -136,9 +145,15 @@ def test_hand_cases(hand_cases):
         U = int(inv.max()) + 1
         cnts = torch.bincount(inv, minlength=U)
         f = torch.from_numpy(c["feats"]).to(DEV)
-        data = T.ScatterData(inv.to(DEV), cnts.to(DEV))
+        data = T.ScatterData(inv.to(DEV), cnts.to(DEV), max_tie_rule="first")
         mx, arg = T.scatter_max(f, data)
         assert bits_equal(mx.cpu().numpy(), c["max"]) and np.array_equal(arg.cpu().numpy(), c["arg"])
+        if "arg_ref" in c:   # grouped rows: the default reports what the reference kernel reports
+            dref = T.ScatterData(inv.to(DEV), cnts.to(DEV))
+            assert dref.is_sorted and dref.max_tie_rule == "reference"
+            mx, arg = T.scatter_max(f, dref)
+            assert np.array_equal(arg.cpu().numpy(), c["arg_ref"]), c["name"]
+            assert bits_equal(mx.cpu().numpy(), c.get("max_ref", c["max"])), c["name"]
         if "sum" in c:
             np.testing.assert_allclose(T.scatter_sum(f, data).cpu().numpy(), c["sum"], rtol=1e-6)
             np.testing.assert_allclose(T.scatter_mean(f, data).cpu().numpy(), c["mean"], rtol=1e-6)
@@ -223,7 +238,9 @@ def test_sorted_input_takes_identity_path_and_matches_unsorted():
     inv[:U] = torch.arange(U)
     feats = torch.randn((N, C), generator=g)
     order = torch.argsort(inv, stable=True)
-    d_sorted = run_case("sorted", feats[order], inv[order], torch.bincount(inv, minlength=U))
+    run_case("sorted_default_rule", feats[order], inv[order], torch.bincount(inv, minlength=U))
+    d_sorted = run_case("sorted", feats[order], inv[order], torch.bincount(inv, minlength=U),
+                        max_tie_rule="first")
     assert d_sorted.perm is None and d_sorted.is_sorted
     d_uns = T.ScatterData(inv.to(DEV), torch.bincount(inv, minlength=U).to(DEV))
     assert d_uns.perm is not None
@@ -339,8 +356,28 @@ def test_lidar_sweep_fp32():
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_lidar_sweep_half(dtype):
-    w = workloads.lidar_sweep(N=400_000, C=128, seed=2)
+    w = workloads.lidar_sweep(N=1_000_000, C=128, seed=2)
     run_case("lidar_sweep_half", w.feats, w.unq_inv, w.unq_cnts, dtype=dtype, grad_seed=102)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_lidar_pillars(dtype):
+    """Unsorted rows, 512-byte (256-byte) rows, and two thirds of the points in voxels that are
+    split across lane groups and merged through LDS and the atomic table."""
+    w = workloads.lidar_pillars()
+    assert int(w.unq_cnts.max()) > 1000 and int((w.unq_cnts > 64).sum()) > 2000
+    data = run_case("lidar_pillars", w.feats, w.unq_inv, w.unq_cnts, dtype=dtype, grad_seed=102)
+    assert data.num_heavy == int((w.unq_cnts > 64).sum())
+
+
+def test_lidar_pillars_grouped_rows():
+    """The same points delivered grouped by voxel, the reference's input contract: the
+    default tie rule is then the reference's (block width 1024 here, several rows per thread
+    in the fullest pillars)."""
+    w = workloads.lidar_pillars()
+    order = torch.sort(w.unq_inv, stable=True)[1]
+    data = run_case("lidar_pillars_grouped", w.feats[order], w.unq_inv[order], w.unq_cnts, grad_seed=102)
+    assert data.max_tie_rule == "reference" and data.max_cnt > 1024
 
 
 def test_zipf_contention():
@@ -524,8 +561,13 @@ def test_reference_tie_rule_mode(sizes):
     mx, arg = T.scatter_max(feats.to(DEV), data)
     assert np.array_equal(arg.cpu().numpy(), want_arg)
     assert bits_equal(mx.cpu().numpy(), want_max)
-    # the default rule on the same data
-    d1 = T.ScatterData(inv.to(DEV), cnts.to(DEV))
+    # grouped rows are the reference's own input: the default reports its winner too
+    d0 = T.ScatterData(inv.to(DEV), cnts.to(DEV))
+    assert d0.max_tie_rule == "reference"
+    mx, arg = T.scatter_max(feats.to(DEV), d0)
+    assert np.array_equal(arg.cpu().numpy(), want_arg) and bits_equal(mx.cpu().numpy(), want_max)
+    # the smallest-row rule on the same data
+    d1 = T.ScatterData(inv.to(DEV), cnts.to(DEV), max_tie_rule="first")
     assert np.array_equal(T.scatter_max(feats.to(DEV), d1)[1].cpu().numpy(), first_arg)
     # all rows through the register path as well (no heavy voxels)
     d2 = T.ScatterData(inv.to(DEV), cnts.to(DEV), heavy_threshold=1 << 20, max_tie_rule="reference")
@@ -537,8 +579,13 @@ def test_reference_tie_rule_mode(sizes):
     scatter_ext.max(feats.to(DEV), data.preSum, out, a, data.max_cnt)
     assert np.array_equal(a.cpu().numpy(), want_arg) and bits_equal(out.cpu().numpy(), want_max)
 
-    # shuffled rows: winner = reference rule on the stably sorted voxel, as original row ids
+    # shuffled rows: the reference defines nothing there and the default is the smallest row
     p = torch.randperm(N, generator=torch.Generator().manual_seed(5))
+    dsh = T.ScatterData(inv[p].to(DEV), cnts.to(DEV))
+    assert dsh.max_tie_rule == "first"
+    assert np.array_equal(T.scatter_max(feats[p].to(DEV), dsh)[1].cpu().numpy(),
+                          orc.scatter_max_first(feats[p].numpy(), inv32[p.numpy()], U)[1])
+    # forced: winner = reference rule on the stably sorted voxel, as original row ids
     want_max_s, want_arg_s = orc.scatter_max_reforder(feats[p].numpy(), inv32[p.numpy()], U)
     ds = T.ScatterData(inv[p].to(DEV), cnts.to(DEV), max_tie_rule="reference")
     mx, arg = T.scatter_max(feats[p].to(DEV).requires_grad_(True), ds)
@@ -555,7 +602,7 @@ def test_reference_tie_rule_mode_matches_default_without_ties():
     T = tx()
     w = workloads.lidar_sweep(N=200_000, C=32, seed=12)
     f = w.feats.to(DEV)
-    a = T.scatter_max(f, T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV)))
+    a = T.scatter_max(f, T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV), max_tie_rule="first"))
     b = T.scatter_max(f, T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV), max_tie_rule="reference"))
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
 
@@ -799,6 +846,31 @@ def test_reference_style_module_calls_reuse_their_plan():
     scatter_ext.sum(f2, pre, out, 100)
     want2 = orc.scatter_sum_f64(feats[:N - 1].numpy(), inv2.numpy().astype(np.int32), U)
     assert np.allclose(out.cpu().numpy(), want2, rtol=1e-5, atol=1e-5)
+    # ... and rewritten in place for another grouping of the SAME number of rows and
+    # voxels: nothing but the contents of preSum tells the two plans apart
+    scatter_ext.clear_csr_plan_cache()
+    scatter_ext.getPreSum(inv.int().to(DEV), pre)
+    out = torch.zeros((U, C), device=DEV)
+    scatter_ext.sum(f, pre, out, int(sizes.max()))           # plan for `sizes` is now cached
+    sizes3 = torch.tensor([1, 1, 2, 70, 5, 9, 130, 3, 1], dtype=torch.long)
+    assert int(sizes3.sum()) == N and sizes3.numel() == U
+    inv3 = torch.repeat_interleave(torch.arange(U), sizes3)
+    scatter_ext.getPreSum(inv3.int().to(DEV), pre)
+    out = torch.zeros((U, C), device=DEV)
+    scatter_ext.sum(f, pre, out, int(sizes3.max()))
+    want3 = orc.scatter_sum_f64(feats.numpy(), inv3.numpy().astype(np.int32), U)
+    assert np.allclose(out.cpu().numpy(), want3, rtol=1e-5, atol=1e-5)
+    wm3, wa3 = orc.scatter_max_reforder(feats.numpy(), inv3.numpy().astype(np.int32), U)
+    mx = torch.zeros((U, C), device=DEV)
+    arg = torch.zeros((U, C), device=DEV, dtype=torch.int32)
+    scatter_ext.max(f, pre, mx, arg, int(sizes3.max()))
+    assert np.array_equal(arg.cpu().numpy(), wa3) and bits_equal(mx.cpu().numpy(), wm3)
+    # a preSum tensor that is gone takes its plan (and the device memory it pins) with it
+    del pre
+    pre4 = torch.zeros(U + 1, dtype=torch.int32, device=DEV)
+    scatter_ext.getPreSum(inv.int().to(DEV), pre4)
+    scatter_ext.sum(f, pre4, torch.zeros((U, C), device=DEV), int(sizes.max()))
+    assert scatter_ext.csr_plan_cache_size() == 1
     scatter_ext.clear_csr_plan_cache()
 
 
@@ -822,3 +894,103 @@ def test_assume_sorted_skips_the_sort_and_is_verified():
     assert torch.equal(T.scatter_mean(f_s, a), T.scatter_mean(f_s, b))
     with pytest.raises(RuntimeError, match="declared sorted"):
         T.ScatterData(w.unq_inv.to(DEV), cnts, assume_sorted=True)
+
+
+# ------------------------------------------- drop-in behaviour on grouped rows --
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_default_scatter_max_on_grouped_tie_heavy_rows_is_the_reference_winner(dtype):
+    """``from torchex import scatter_max, ScatterData`` on rows grouped by voxel -- the only
+    input the reference defines -- reports the row the reference kernel reports, also where
+    many rows tie (values 0, 1, 2 only; block widths 32 .. 1024, several rows per thread)."""
+    import torchex
+    sizes = [5, 17, 31, 32, 33, 64, 1, 2, 100, 7, 700, 1024, 900, 65, 2050, 1500, 40, 4996, 1025, 3000] * 3
+    C = 24
+    feats, inv, cnts = _tie_heavy_groups(77, sizes, C)
+    U = len(sizes)
+    inv32 = inv.numpy().astype(np.int32)
+    want_max, want_arg = orc.scatter_max_reforder(feats.numpy(), inv32, U)
+    assert (want_arg != orc.scatter_max_first(feats.numpy(), inv32, U)[1]).any()
+    data = torchex.ScatterData(inv.to(DEV), cnts.to(DEV))
+    mx, arg = torchex.scatter_max(feats.to(dtype).to(DEV), data)
+    assert mx.dtype == dtype
+    assert np.array_equal(arg.cpu().numpy(), want_arg)
+    assert bits_equal(mx.float().cpu().numpy(), want_max)
+
+
+def test_reference_harness_form_with_torch_timer(capsys):
+    """The reference's own test loop (test/test_scatter.py:27-51): ScatterData built outside
+    the timers, ``with timer.timing(name)`` around each operator call, running means printed
+    every ``freq`` calls; all three modes (the reference enables 'sum' only), checked against
+    the closed forms of its data instead of torch_scatter."""
+    from torchex import ScatterData, TorchTimer, scatter_max, scatter_mean, scatter_sum
+    freq = 5
+    timer_torchex = TorchTimer(freq)
+    w = workloads.reference_test_groups(channel=128, num_group=60)
+    feat, unq_inv, unq_cnts = w.feats.to(DEV), w.unq_inv.to(DEV), w.unq_cnts.to(DEV)
+    data = ScatterData(unq_inv, unq_cnts)
+    n = w.unq_cnts.double().unsqueeze(1)
+    starts = torch.cumsum(w.unq_cnts, 0) - w.unq_cnts
+    col = w.feats[:, 0]
+    argpos = torch.stack([s + torch.argmax(col[s:s + c]) for s, c in zip(starts.tolist(), w.unq_cnts.tolist())])
+    for mode in ("sum", "mean", "max"):
+        for _ in range(2 * freq):
+            with timer_torchex.timing(f"Torchex.scatter_{mode}"):
+                if mode == "sum":
+                    ans2 = scatter_sum(feat, data)
+                elif mode == "mean":
+                    ans2 = scatter_mean(feat, data)
+                else:
+                    ans2, arg2 = scatter_max(feat, data)
+            want = {"sum": n * (n - 1) / 2, "mean": (n - 1) / 2, "max": n - 1}[mode]
+            assert torch.equal(ans2.cpu().double(), want.expand(-1, 128))
+            if mode == "max":
+                assert torch.equal(arg2.cpu().long(), argpos.unsqueeze(1).expand(-1, 128))
+    lines = [l for l in capsys.readouterr().out.splitlines() if l.startswith("Average time cost of Torchex.")]
+    assert len(lines) == 6                      # 3 modes x (10 calls / freq 5)
+    for l in lines:
+        assert l.endswith("ms") and float(l.split(": ")[1][:-2]) > 0.0
+    t = timer_torchex.timer_dict["Torchex.scatter_max"]
+    assert t.exe_counter == 0 and t.print_freq == freq     # reset after each print
+
+
+def test_get_presum_against_the_reference_restatement():
+    """scatter_ext.getPreSum / getPreSum() against the oracle's restatement of the reference
+    kernel (scatter_kernel.cu:85-100), including a tail of equal ids and single-row groups."""
+    import scatter_ext
+    T = tx()
+    rs = np.random.RandomState(3)
+    for sizes in ([1], [5], [1, 1, 1], [3, 1, 70, 2, 5, 130, 1, 1, 9], rs.randint(1, 400, size=3000).tolist()):
+        inv = np.repeat(np.arange(len(sizes)), sizes).astype(np.int32)
+        want = orc.get_presum_ref(inv)
+        pre = torch.zeros(len(sizes) + 1, dtype=torch.int32, device=DEV)
+        scatter_ext.getPreSum(torch.from_numpy(inv).to(DEV), pre)
+        assert np.array_equal(pre.cpu().numpy(), want)
+        assert np.array_equal(T.getPreSum(torch.from_numpy(inv).long().to(DEV)).cpu().numpy(), want)
+
+
+def test_concurrent_streams_do_not_share_a_heavy_voxel_table():
+    """Forwards of one ScatterData queued on two streams at the same time: each stream gets a
+    heavy-voxel table of its own, so the results equal the single-stream ones."""
+    T = tx()
+    w = workloads.zipf_contention(N=400_000, C=32, num_ids=300, seed=5)     # every voxel heavy
+    inv, cnts = w.unq_inv.to(DEV), w.unq_cnts.to(DEV)
+    fa = w.feats.to(DEV)
+    fb = (w.feats * 0.5 + 1.0).to(DEV)
+    data = T.ScatterData(inv, cnts)
+    assert data.num_heavy == w.U
+    ref_a, ref_b = T.scatter_max(fa, data), T.scatter_max(fb, data)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs_a, outs_b = [], []
+    for _ in range(6):
+        with torch.cuda.stream(s1):
+            outs_a.append(T.scatter_max(fa, data))
+        with torch.cuda.stream(s2):
+            outs_b.append(T.scatter_max(fb, data))
+    torch.cuda.synchronize()
+    for mx, arg in outs_a:
+        assert torch.equal(mx, ref_a[0]) and torch.equal(arg, ref_a[1])
+    for mx, arg in outs_b:
+        assert torch.equal(mx, ref_b[0]) and torch.equal(arg, ref_b[1])
+    assert len(data._scratch) == 3 and all(not bool((t != 0).any()) for t in data._scratch.values())

@@ -123,6 +123,11 @@ def test_hand_cases(hand_cases):
         m, a = orc.scatter_max_first(feats, inv, U)
         assert_bits_equal(m, c["max"]), c["name"]
         assert np.array_equal(a, c["arg"]), c["name"]
+        if "arg_ref" in c:   # grouped rows: what the reference kernel itself reports
+            assert np.all(np.diff(inv) >= 0)
+            mr, ar = orc.scatter_max_ref(feats, orc.presum(cnt), int(cnt.max()))
+            assert np.array_equal(ar, c["arg_ref"]), c["name"]
+            assert_bits_equal(mr, c.get("max_ref", c["max"])), c["name"]
         if "sum" in c:
             s64 = orc.scatter_sum_f64(feats, inv, U)
             np.testing.assert_allclose(s64, c["sum"], rtol=1e-6, atol=0)

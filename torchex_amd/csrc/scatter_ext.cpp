@@ -407,13 +407,20 @@ Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const 
 // The reference module's entry points take only CSR offsets, every call.  The plan that
 // goes with a preSum tensor is kept for the next calls (the reference's ScatterData
 // makes preSum once and then calls sum/max many times): a few entries, keyed by the
-// tensor's storage, length and version, each holding the tensor itself so that its
-// storage cannot be handed to another tensor while the entry lives.
+// tensor object, its memory, length and version counter.
 struct CsrPlan {
-    Tensor preSum, seg, slot_of, heavy_ids;
+    // The preSum tensor the plan was built from, held weakly: the entry dies with the
+    // tensor (so the cache pins device memory only for tensors still in use) and a later
+    // tensor that happens to get the same address can never match it.
+    c10::weak_intrusive_ptr<c10::TensorImpl> owner;
+    const void *data = nullptr;
+    Tensor seg, slot_of, heavy_ids;
     uint32_t version = 0;
-    int64_t num_total = 0, num_heavy = 0;
-    std::vector<std::pair<int64_t, Tensor>> scratch;  // per channel count
+    int64_t numel = 0, num_total = 0, num_heavy = 0;
+    // zeroed heavy-voxel tables, one per (channel count, stream): calls on one stream are
+    // ordered, calls on different streams must not share a table
+    std::vector<std::tuple<int64_t, void *, Tensor>> scratch;
+    explicit CsrPlan(const Tensor &preSum) : owner(preSum.getIntrusivePtr()) {}
 };
 constexpr size_t kCsrPlanCacheSize = 8;
 std::vector<CsrPlan> &csr_plan_cache() {
@@ -423,20 +430,43 @@ std::vector<CsrPlan> &csr_plan_cache() {
     return *cache;
 }
 
+void drop_orphaned_csr_plans() {
+    auto &cache = csr_plan_cache();
+    cache.erase(std::remove_if(cache.begin(), cache.end(), [](const CsrPlan &p) { return p.owner.expired(); }),
+                cache.end());
+}
+
+// Plans built from memory that `preSum` covers are void once it is rewritten (getPreSum
+// writes through a raw pointer).
+void drop_csr_plans_of(const Tensor &preSum) {
+    auto &cache = csr_plan_cache();
+    const char *lo = (const char *)preSum.data_ptr();
+    const char *hi = lo + preSum.numel() * (int64_t)sizeof(int32_t);
+    cache.erase(std::remove_if(cache.begin(), cache.end(),
+                               [&](const CsrPlan &p) {
+                                   const char *a = (const char *)p.data;
+                                   const char *b = a + p.numel * (int64_t)sizeof(int32_t);
+                                   return p.owner.expired() || (a < hi && lo < b);
+                               }),
+                cache.end());
+}
+
 CsrPlan &csr_plan_for(const Tensor &preSum, int64_t num_total) {
     auto &cache = csr_plan_cache();
+    drop_orphaned_csr_plans();
     const uint32_t version = preSum.unsafeGetTensorImpl()->version_counter().current_version();
     for (size_t i = 0; i < cache.size(); ++i) {
         CsrPlan &p = cache[i];
-        if (p.preSum.data_ptr() == preSum.data_ptr() && p.preSum.numel() == preSum.numel() &&
-            p.preSum.device() == preSum.device() && p.version == version && p.num_total == num_total) {
+        if (p.owner._unsafe_get_target() == preSum.unsafeGetTensorImpl() && p.data == preSum.data_ptr() &&
+            p.numel == preSum.numel() && p.version == version && p.num_total == num_total) {
             if (i != 0) std::rotate(cache.begin(), cache.begin() + i, cache.begin() + i + 1);  // most recent first
             return cache.front();
         }
     }
     auto [seg, slot_of, heavy_ids, hs] = plan_from_presum(preSum, num_total, txs_default_heavy_threshold());
-    CsrPlan p;
-    p.preSum = preSum;
+    CsrPlan p(preSum);
+    p.data = preSum.data_ptr();
+    p.numel = preSum.numel();
     p.seg = seg;
     p.slot_of = slot_of;
     p.heavy_ids = heavy_ids;
@@ -456,20 +486,33 @@ void csr_reduce(int op, Tensor feats, Tensor preSum, Tensor out, OptTensor arg, 
     TORCH_CHECK(out.scalar_type() == feats.scalar_type(), "out dtype must match feats");
     TORCH_CHECK(preSum.numel() == out.size(0) + 1, "preSum must have out.size(0)+1 entries");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(feats.device());
-    CsrPlan &plan = csr_plan_for(preSum, feats.size(0));
     const int64_t C = feats.size(1);
-    Tensor scratch;
-    for (auto &kv : plan.scratch)
-        if (kv.first == C) scratch = kv.second;
-    if (!scratch.defined()) {
-        scratch = make_scratch(plan.num_heavy, C, feats);
-        plan.scratch.emplace_back(C, scratch);
+    void *st = cur_stream(feats);
+    // Everything the launch needs is copied out of the cache entry (tensor handles, by
+    // value) while the GIL is held: run_forward releases it, and another Python thread
+    // may then insert into or reorder the cache.
+    Tensor seg, slot_of, heavy_ids, scratch;
+    {
+        CsrPlan &plan = csr_plan_for(preSum, feats.size(0));
+        for (auto &entry : plan.scratch)
+            if (std::get<0>(entry) == C && std::get<1>(entry) == st) scratch = std::get<2>(entry);
+        if (!scratch.defined()) {
+            scratch = make_scratch(plan.num_heavy, C, feats);
+            plan.scratch.emplace_back(C, st, scratch);
+        }
+        seg = plan.seg;
+        slot_of = plan.slot_of;
+        heavy_ids = plan.heavy_ids;
     }
     OptTensor perm;
-    run_forward(op, feats, perm, plan.seg, preSum, plan.slot_of, plan.heavy_ids, scratch, out, arg, max_cnt);
+    run_forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, out, arg, max_cnt);
 }
 
 void clear_csr_plan_cache() { csr_plan_cache().clear(); }
+int64_t csr_plan_cache_size() {
+    drop_orphaned_csr_plans();
+    return (int64_t)csr_plan_cache().size();
+}
 
 // sum(feats, preSum, out, max_cnt): max_cnt only shaped the reference's thread
 // blocks (scatter_kernel.cu:179); it does not change a sum and is not needed here.
@@ -493,6 +536,11 @@ void get_presum_ref(Tensor unq_inv, Tensor preSum) {
     check_status(txs_get_presum(i32p(unq_inv), i32w(preSum), unq_inv.numel(), preSum.numel(),
                                 cur_stream(unq_inv)),
                  "getPreSum");
+    // preSum was rewritten through a raw pointer: say so to autograd's version counter
+    // (the plans kept for sum/max are keyed on it) and drop the plans built from the old
+    // contents of this storage
+    preSum.unsafeGetTensorImpl()->bump_version();
+    drop_csr_plans_of(preSum);
 }
 
 }  // namespace
@@ -513,6 +561,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("grid_hash_probe", &grid_hash_probe, "probe_table(coors, table) -> values");
     m.def("make_scratch", &make_scratch, "zeroed scratch table, one row per heavy voxel");
     m.def("clear_csr_plan_cache", &clear_csr_plan_cache, "drop the plans kept for sum/max over CSR offsets");
+    m.def("csr_plan_cache_size", &csr_plan_cache_size, "number of plans currently kept for sum/max over CSR offsets");
     m.def("forward", &forward, "forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, max_cnt)");
     m.def("backward", &backward, "backward(op, grad_out, arg, perm, seg, preSum, num_total)");
     m.def("abi_version", &txs_abi_version);

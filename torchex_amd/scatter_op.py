@@ -12,6 +12,12 @@ bundles the index data once per voxelization, and ``scatter_sum`` /
   written; the intended ``zeros.scatter_(0, arg, g)`` is what runs here);
 * ``scatter_mean`` is one fused kernel rather than sum followed by a divide.
 
+Which row ``scatter_max`` reports among equal maxima: when ``unq_inv`` arrives
+grouped by voxel -- the only order the reference accepts (``scatter_op.py:18-19``) --
+the row the reference kernel itself reports (``scatter_kernel.cu:41-83,146-152``), so a
+program written for the reference sees the same ``arg``; for any other order, where the
+reference is undefined, the smallest row index.  ``max_tie_rule`` forces either.
+
 There is no PyTorch fallback: everything runs in the HIP kernels behind
 ``scatter_ext``.
 """
@@ -21,6 +27,21 @@ from torch.autograd import Function
 from ._native import scatter_ext
 
 _SUM, _MEAN, _MAX = scatter_ext.SUM, scatter_ext.MEAN, scatter_ext.MAX
+
+
+def _check_tie_rule(rule):
+    if rule not in (None, "first", "reference"):
+        raise ValueError("max_tie_rule must be None, 'first' or 'reference'")
+
+
+def _resolve_tie_rule(rule, grouped):
+    """Which row scatter_max reports among equal maxima.  ``None`` (the default) means:
+    the reference kernel's own winner when the rows arrived grouped by voxel, which is
+    the only input the reference defines (scatter_op.py:18-19), and the smallest row
+    index otherwise."""
+    if rule is None:
+        return "reference" if grouped else "first"
+    return rule
 
 
 class ScatterData:
@@ -34,12 +55,17 @@ class ScatterData:
     voxel at each sorted position, bit 31 marking voxels reduced through
     atomics), ``slot_of`` / ``heavy_ids`` (table of those voxels).
 
+    ``max_tie_rule``: ``"reference"`` reports, among equal maxima, the row the reference
+    kernel reports for the voxel's rows taken in ascending order; ``"first"`` the
+    smallest row index; ``None`` (default) picks ``"reference"`` for grouped input and
+    ``"first"`` otherwise.  The rule in force is kept as ``self.max_tie_rule``.
+
     ``assume_sorted=True`` states that ``unq_inv`` is already grouped (the order the
     reference requires): the sort is then not queued at all; the statement is
     verified on the device and an unsorted ``unq_inv`` raises.
     """
 
-    def __init__(self, unq_inv, unq_cnts, heavy_threshold=None, max_tie_rule="first",
+    def __init__(self, unq_inv, unq_cnts, heavy_threshold=None, max_tie_rule=None,
                  assume_sorted=False) -> None:
         assert unq_inv.ndim in (
             1, 2), f"unq_inv in ScatterData should be 1 or 2-dims, but got {unq_inv.ndim}-dims"
@@ -50,11 +76,7 @@ class ScatterData:
             self.unq_cnts = unq_cnts.unsqueeze(-1)
         else:
             self.unq_cnts = unq_cnts
-        if max_tie_rule not in ("first", "reference"):
-            raise ValueError("max_tie_rule must be 'first' or 'reference'")
-        # which row scatter_max reports among equal maxima: the smallest row
-        # index, or the row the reference kernel's shuffle tree would keep
-        self.max_tie_rule = max_tie_rule
+        _check_tie_rule(max_tie_rule)
         if heavy_threshold is None:
             heavy_threshold = scatter_ext.default_heavy_threshold()
         self.heavy_threshold = int(heavy_threshold)
@@ -68,6 +90,7 @@ class ScatterData:
         assert stats[5] == 0, "unq_cnts is not the histogram of unq_inv"
         self.num_total = flat.shape[0]
         self.is_sorted = self.perm is None
+        self.max_tie_rule = _resolve_tie_rule(max_tie_rule, self.is_sorted)
         self.max_cnt = int(stats[2])
         self.num_special = int(stats[3])
         self.num_heavy = int(stats[7])
@@ -75,16 +98,14 @@ class ScatterData:
         self._scratch = {}
 
     @classmethod
-    def from_keys(cls, keys, key_bound, heavy_threshold=None, max_tie_rule="first", _stats=None):
+    def from_keys(cls, keys, key_bound, heavy_threshold=None, max_tie_rule=None, _stats=None):
         """ScatterData straight from voxel keys (any non-negative int ids below
         ``key_bound``, e.g. linear voxel ids): computes what ``torch.unique(keys,
         return_inverse=True, return_counts=True)`` returns -- kept as ``unq_keys``,
         ``unq_inv``, ``unq_cnts`` -- and the scatter plan from ONE sort of the keys,
         where ``torch.unique`` followed by ``ScatterData(...)`` sorts twice."""
-        if max_tie_rule not in ("first", "reference"):
-            raise ValueError("max_tie_rule must be 'first' or 'reference'")
+        _check_tie_rule(max_tie_rule)
         self = cls.__new__(cls)
-        self.max_tie_rule = max_tie_rule
         if heavy_threshold is None:
             heavy_threshold = scatter_ext.default_heavy_threshold()
         self.heavy_threshold = int(heavy_threshold)
@@ -97,6 +118,7 @@ class ScatterData:
         self.unq_cnts = cnts.unsqueeze(-1)
         self.num_total = flat.shape[0]
         self.is_sorted = self.perm is None
+        self.max_tie_rule = _resolve_tie_rule(max_tie_rule, self.is_sorted)
         self.max_cnt = int(stats[2])
         self.num_special = int(stats[3])
         self.num_heavy = int(stats[7])
@@ -105,7 +127,7 @@ class ScatterData:
         return self
 
     @classmethod
-    def from_points(cls, points, voxel_size, pc_range, heavy_threshold=None, max_tie_rule="first"):
+    def from_points(cls, points, voxel_size, pc_range, heavy_threshold=None, max_tie_rule=None):
         """Dynamic voxelization in one go: voxel coordinates as the reference's
         ``voxelize_single`` computes them (``test/test_incremental_mask.py:20-26``),
         x-major linear keys (``operator_py/incremental_points.py:18-19``), unique and
@@ -119,14 +141,14 @@ class ScatterData:
 
     def scratch(self, channel):
         """Zeroed table the heavy voxels are merged in (one row each); the kernels leave it
-        zeroed again, so one buffer per channel count is kept for reuse.  Forward
-        calls that share a ``ScatterData`` therefore must not overlap in time on the
-        GPU (two streams running them concurrently would race on this table); calls
-        on one stream, the normal case, are ordered."""
-        buf = self._scratch.get(channel)
+        zeroed again, so a buffer is kept for reuse -- one per channel count and per
+        stream: calls queued on one stream are ordered, and forwards that run
+        concurrently on different streams each get a table of their own."""
+        key = (channel, torch.cuda.current_stream(self.seg.device).stream_id)
+        buf = self._scratch.get(key)
         if buf is None:
             buf = scatter_ext.make_scratch(self.num_heavy, channel, self.seg)
-            self._scratch[channel] = buf
+            self._scratch[key] = buf
         return buf
 
 
@@ -192,9 +214,9 @@ class ScatterMaxFunction(Function):
         """scatter_max forward (``scatter_op.py:84-103``).
         Returns ``(out [num_unq, channel], arg [num_unq, channel] int32)`` where
         ``arg`` is the row index into ``feats`` of the winning element.  When
-        several rows tie, the smallest row wins (``data.max_tie_rule ==
-        "first"``, the default) or the row the reference kernel would report
-        for the voxel's rows in ascending order (``"reference"``).
+        several rows tie, ``data.max_tie_rule`` decides: ``"reference"`` (the
+        default for grouped ``unq_inv``) reports the row the reference kernel
+        reports, ``"first"`` (the default for any other order) the smallest row.
         """
         op = scatter_ext.MAX_REFTIE if data.max_tie_rule == "reference" else _MAX
         out, arg = _forward(op, feats, data)
