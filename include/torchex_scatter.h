@@ -6,7 +6,8 @@
  * (a hipStream_t passed as void*; NULL = the null stream) and an int status.
  * No torch type crosses this line.  The library allocates no device memory:
  * every buffer, workspaces included, is owned by the caller.  Calls are
- * asynchronous on `stream` and re-entrant (no global state).
+ * asynchronous on `stream` and re-entrant (no global state), with one exception
+ * that says so: txs_scatter_forward_resident, which uses a table inside the library.
  *
  * Each entry point names the reference interface it stands in for
  * (paths relative to the TorchEx tree).
@@ -46,7 +47,13 @@
 extern "C" {
 #endif
 
-enum { TXS_OK = 0, TXS_ERR_INVALID_ARG = 1, TXS_ERR_LAUNCH = 2, TXS_ERR_UNSUPPORTED = 3 };
+enum {
+    TXS_OK = 0,
+    TXS_ERR_INVALID_ARG = 1,
+    TXS_ERR_LAUNCH = 2,
+    TXS_ERR_UNSUPPORTED = 3,
+    TXS_ERR_TOO_LARGE = 4 /* txs_scatter_forward_resident: num_heavy * channel exceeds the resident table */
+};
 enum { TXS_F32 = 0, TXS_F16 = 1, TXS_BF16 = 2 };
 enum { TXS_SUM = 0, TXS_MEAN = 1, TXS_MAX = 2, TXS_MAX_REFTIE = 3 };
 
@@ -63,7 +70,7 @@ enum {
     TXS_STATS_LEN = 8
 };
 
-/* Library ABI version (6); bumped when a signature or the meaning of an argument changes. */
+/* Library ABI version (7); bumped when a signature or the meaning of an argument changes. */
 int txs_abi_version(void);
 
 /* Human-readable text for a status code. */
@@ -225,6 +232,32 @@ int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *per
                         const int32_t *heavy_ids, int64_t num_special, void *scratch,
                         void *out, int32_t *arg, int64_t num_total, int64_t channel,
                         int64_t num_unq, int64_t max_cnt, void *stream);
+
+/* txs_scatter_forward for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments and results as txs_scatter_forward,
+ * except that the heavy-voxel table is not passed in: the call uses a table that
+ * lives in the library's own device image (one copy per GPU, 8 MiB, held until the
+ * process ends), and num_heavy (TXS_STAT_NUM_HEAVY of the plan) says how many rows of
+ * it are needed.  The call allocates and frees nothing and only launches kernels: it
+ * clears the num_heavy * channel cells it is going to use, then runs the same kernels
+ * as txs_scatter_forward.
+ *   Limit: num_heavy * channel <= txs_resident_table_cells() (1,048,576 cells, e.g.
+ *   8192 heavy voxels of 128 channels); beyond it the call returns TXS_ERR_TOO_LARGE
+ *   and launches nothing.
+ *   Every call on one GPU shares that GPU's table: two calls that overlap in time on
+ *   one GPU (different streams, or different host threads) race.  Calls queued on one
+ *   stream are ordered and safe.
+ *   The device that owns `stream` must be current.  The table's address is looked up
+ *   the first time the call runs on a GPU; txs_resident_table_init() does that lookup
+ *   ahead of time for the current GPU (call it before a graph capture starts). */
+int txs_scatter_forward_resident(int op, int dtype, const void *feats, const int32_t *perm,
+                                 const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
+                                 const int32_t *heavy_ids, int64_t num_special, int64_t num_heavy,
+                                 void *out, int32_t *arg, int64_t num_total, int64_t channel,
+                                 int64_t num_unq, int64_t max_cnt, void *stream);
+int txs_resident_table_init(void);
+int64_t txs_resident_table_cells(void);
 
 /* Backward as one gather pass over the sorted positions.  Replaces the ATen
  * ops of ScatterSumFunction.backward (scatter_op.py:47-50: g[unq_inv]),

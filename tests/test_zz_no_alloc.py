@@ -1,0 +1,96 @@
+"""The forward entry point that allocates nothing (``txs_scatter_forward_resident``: the
+heavy-voxel table lives inside the library) against ``txs_scatter_forward`` with a
+caller-owned table, through the C ABI on raw device pointers.  Two calls in a row, the
+second on a smaller input, so that whatever the first call left in the shared table
+would show.  Max / argmax bit-exact; sum within 1e-5 of the summand scale (the two calls
+add the same partials in a different atomic order)."""
+import ctypes
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as orc
+from torchex_amd import workloads
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+SUM, MEAN, MAX = 0, 1, 2
+F32 = 0
+
+
+def _say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def _forward(lib, resident, op, f, data, stream):
+    import torchex_amd  # noqa: F401
+    N, C = f.shape
+    U = data.num_unq
+    vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    out = torch.full((U, C), 7.0, device=DEV)
+    arg = torch.full((U, C), -7, device=DEV, dtype=torch.int32)
+    perm = vp(data.perm.data_ptr()) if data.perm is not None else vp(0)
+    heavy = vp(data.heavy_ids.data_ptr() if data.num_special else 0)
+    common_head = (ci(op), ci(F32), vp(f.data_ptr()), perm, vp(data.seg.data_ptr()), vp(data.preSum.data_ptr()),
+                   vp(data.slot_of.data_ptr()), heavy, i64(data.num_special))
+    common_tail = (vp(out.data_ptr()), vp(arg.data_ptr()), i64(N), i64(C), i64(U), i64(data.max_cnt), stream)
+    if resident:
+        lib.txs_scatter_forward_resident.restype = ctypes.c_int
+        rc = lib.txs_scatter_forward_resident(*common_head, i64(data.num_heavy), *common_tail)
+        table = None
+    else:
+        table = torch.zeros((max(data.num_heavy, 1) * C,), device=DEV, dtype=torch.int64)
+        lib.txs_scatter_forward.restype = ctypes.c_int
+        rc = lib.txs_scatter_forward(*common_head, vp(table.data_ptr()), *common_tail)
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    return out, arg
+
+
+def test_resident_table_forward_matches_caller_table_forward():
+    from torchex_amd import _native
+    import torchex_amd as T
+    lib = _native.cabi()
+    lib.txs_resident_table_cells.restype = ctypes.c_int64
+    cap = lib.txs_resident_table_cells()
+    assert cap == 1 << 20
+    assert lib.txs_resident_table_init() == 0
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    big = workloads.lidar_pillars(N=300_000, C=64, seed=3)       # hundreds of heavy voxels
+    small = workloads.zipf_contention(N=60_000, C=64, num_ids=40, seed=6)   # fewer, all heavy
+    for w in (big, small):
+        _say(f"[case] resident table {w.name} N={w.N} C={w.C} U={w.U}")
+        f = w.feats.to(DEV)
+        data = T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV))
+        assert 0 < data.num_heavy and data.num_heavy * w.C <= cap
+        inv32 = w.unq_inv.numpy().astype(np.int32)
+        sabs = orc.scatter_sum_f64(np.abs(w.feats.numpy()), inv32, w.U)
+        for op in (MAX, SUM, MEAN, MAX):
+            a_out, a_arg = _forward(lib, False, op, f, data, stream)
+            b_out, b_arg = _forward(lib, True, op, f, data, stream)
+            if op == MAX:
+                assert torch.equal(a_arg, b_arg) and torch.equal(a_out, b_out)
+                wm, wa = orc.scatter_max_first(w.feats.numpy(), inv32, w.U)
+                assert np.array_equal(b_arg.cpu().numpy(), wa) and np.array_equal(b_out.cpu().numpy(), wm)
+            else:
+                scale = sabs / (w.unq_cnts.numpy()[:, None] if op == MEAN else 1.0)
+                d = np.abs(a_out.cpu().numpy().astype(np.float64) - b_out.cpu().numpy())
+                assert np.all(d <= 1e-5 * scale)
+                light = (w.unq_cnts <= data.heavy_threshold).to(DEV)
+                assert torch.equal(a_out[light], b_out[light])   # register path: same order, same bits
+    # beyond the table's capacity: a clear status, nothing launched
+    wide = workloads.zipf_contention(N=300_000, C=8, num_ids=200, seed=7)
+    data = T.ScatterData(wide.unq_inv.to(DEV), wide.unq_cnts.to(DEV))
+    vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    out = torch.full((wide.U, 8), 7.0, device=DEV)
+    lib.txs_scatter_forward_resident.restype = ctypes.c_int
+    rc = lib.txs_scatter_forward_resident(
+        ci(SUM), ci(F32), vp(1), vp(0), vp(1), vp(1), vp(1), vp(1), i64(2_000_000), i64(2_000_000),
+        vp(out.data_ptr()), vp(0), i64(10), i64(8), i64(2_000_000), i64(1), stream)
+    assert rc == 4
+    lib.txs_status_string.restype = ctypes.c_char_p
+    assert b"exceeds" in lib.txs_status_string(4)
+    torch.cuda.synchronize()
+    assert bool((out == 7.0).all())

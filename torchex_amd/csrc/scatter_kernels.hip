@@ -27,6 +27,16 @@
 
 #include "txs_common.h"
 
+#include <mutex>
+
+// Heavy-voxel table that lives in the library's own device image, for callers that cannot
+// allocate device memory (code under HIP graph capture, tight serving loops): one copy
+// per GPU, 8 MiB each, held until the process ends.  Host code never passes this name to
+// a kernel: the device address is looked up once per GPU (resident_table() below) and
+// that pointer is what kernels and the clearing launch receive.
+constexpr long long kResidentCells = 1LL << 20;
+static __device__ __align__(256) unsigned long long static_scratch[kResidentCells];
+
 namespace {
 
 // ----------------------------------------------------------------- forward --
@@ -756,32 +766,13 @@ hipError_t launch_bwd(int op, const Geometry &geo, hipStream_t st, const void *g
     return hipErrorInvalidValue;
 }
 
-}  // namespace
-
-// =================================================================== C ABI ==
-
-extern "C" {
-
-int txs_abi_version(void) { return 6; }
-
-const char *txs_status_string(int status) {
-    switch (status) {
-        case TXS_OK: return "ok";
-        case TXS_ERR_INVALID_ARG: return "invalid argument (null pointer, negative or oversized extent)";
-        case TXS_ERR_LAUNCH: return "HIP kernel launch failed";
-        case TXS_ERR_UNSUPPORTED: return "unsupported dtype or operator";
-        default: return "unknown status";
-    }
-}
-
-int txs_default_heavy_threshold(void) { return kHeavyDefault; }
-int txs_chunk_rows(void) { return kChunk; }
-
-int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *perm,
-                        const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
-                        const int32_t *heavy_ids, int64_t num_special, void *scratch, void *out,
-                        int32_t *arg, int64_t num_total, int64_t channel, int64_t num_unq,
-                        int64_t max_cnt, void *stream) {
+// Argument checks and the two launches (reduction, then the special voxels' rows) behind
+// txs_scatter_forward and txs_scatter_forward_resident.
+int scatter_forward_impl(int op, int dtype, const void *feats, const int32_t *perm,
+                         const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
+                         const int32_t *heavy_ids, int64_t num_special, void *scratch, void *out,
+                         int32_t *arg, int64_t num_total, int64_t channel, int64_t num_unq,
+                         int64_t max_cnt, void *stream) {
     if (op != TXS_SUM && op != TXS_MEAN && op != TXS_MAX && op != TXS_MAX_REFTIE)
         return TXS_ERR_UNSUPPORTED;
     if (dtype != TXS_F32 && dtype != TXS_F16 && dtype != TXS_BF16) return TXS_ERR_UNSUPPORTED;
@@ -821,6 +812,38 @@ int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *per
     return status_of(e);
 }
 
+}  // namespace
+
+// =================================================================== C ABI ==
+
+extern "C" {
+
+int txs_abi_version(void) { return 7; }
+
+const char *txs_status_string(int status) {
+    switch (status) {
+        case TXS_OK: return "ok";
+        case TXS_ERR_INVALID_ARG: return "invalid argument (null pointer, negative or oversized extent)";
+        case TXS_ERR_LAUNCH: return "HIP kernel launch failed";
+        case TXS_ERR_UNSUPPORTED: return "unsupported dtype or operator";
+        case TXS_ERR_TOO_LARGE:
+            return "heavy-voxel table (num_heavy * channel cells) exceeds the library's resident table";
+        default: return "unknown status";
+    }
+}
+
+int txs_default_heavy_threshold(void) { return kHeavyDefault; }
+int txs_chunk_rows(void) { return kChunk; }
+
+int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *perm,
+                        const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
+                        const int32_t *heavy_ids, int64_t num_special, void *scratch, void *out,
+                        int32_t *arg, int64_t num_total, int64_t channel, int64_t num_unq,
+                        int64_t max_cnt, void *stream) {
+    return scatter_forward_impl(op, dtype, feats, perm, seg, preSum, slot_of, heavy_ids, num_special,
+                                scratch, out, arg, num_total, channel, num_unq, max_cnt, stream);
+}
+
 int txs_scatter_backward(int op, int dtype, const void *grad_out, const int32_t *arg,
                          const int32_t *perm, const int32_t *seg, const int32_t *preSum,
                          void *grad_in, int64_t num_total, int64_t channel, int64_t num_unq,
@@ -847,6 +870,70 @@ int txs_scatter_backward(int op, int dtype, const void *grad_out, const int32_t 
     else
         e = launch_bwd<BF16>(op, geo, st, grad_out, arg, perm, seg, preSum, grad_in, N, C, U);
     return status_of(e);
+}
+
+}  // extern "C"
+
+// ------------------------------------------------ library-resident heavy table --
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_resident_mu;
+unsigned long long *g_resident_ptr[kMaxDevices];  // device address of static_scratch on each GPU
+
+// Address of the current GPU's copy of static_scratch, looked up on first use.
+int resident_table(unsigned long long **table) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return TXS_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(g_resident_mu);
+    if (g_resident_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch)) != hipSuccess || p == nullptr)
+            return TXS_ERR_LAUNCH;
+        g_resident_ptr[dev] = static_cast<unsigned long long *>(p);
+    }
+    *table = g_resident_ptr[dev];
+    return TXS_OK;
+}
+
+__global__ void clear_cells_kernel(unsigned long long *__restrict__ cells, long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) cells[i] = 0ull;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t txs_resident_table_cells(void) { return kResidentCells; }
+
+int txs_resident_table_init(void) {
+    unsigned long long *table = nullptr;
+    return resident_table(&table);
+}
+
+int txs_scatter_forward_resident(int op, int dtype, const void *feats, const int32_t *perm,
+                                 const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
+                                 const int32_t *heavy_ids, int64_t num_special, int64_t num_heavy,
+                                 void *out, int32_t *arg, int64_t num_total, int64_t channel,
+                                 int64_t num_unq, int64_t max_cnt, void *stream) {
+    if (!fits_i32(channel) || !fits_i32(num_unq) || num_heavy < 0 || num_heavy > num_special ||
+        num_special > num_unq)
+        return TXS_ERR_INVALID_ARG;
+    const int64_t cells = num_heavy * channel;  // both below 2^31: no overflow
+    if (cells > kResidentCells) return TXS_ERR_TOO_LARGE;
+    unsigned long long *table = nullptr;
+    if (cells > 0) {
+        const int rc = resident_table(&table);
+        if (rc != TXS_OK) return rc;
+        // the table is shared by every call on this GPU and keeps what the last one left:
+        // clear the part this call uses (a kernel, so that the call can be captured)
+        clear_cells_kernel<<<dim3(blocks_for(cells)), dim3(kThreads), 0, (hipStream_t)stream>>>(table, cells);
+        if (hipGetLastError() != hipSuccess) return TXS_ERR_LAUNCH;
+    }
+    return scatter_forward_impl(op, dtype, feats, perm, seg, preSum, slot_of, heavy_ids, num_special,
+                                table, out, arg, num_total, channel, num_unq, max_cnt, stream);
 }
 
 }  // extern "C"
