@@ -5,8 +5,8 @@ A "step" is one pass of the hot path over one batch of synthetic points:
 ``scatter_mean`` forward+backward and ``scatter_max`` (+argmax) forward+backward,
 through the public Python API (autograd included), with ``ScatterData`` built
 beforehand (the reference's own timing also keeps ``ScatterData`` construction
-outside the timed region, ``test/test_scatter.py:24,38-44``).  The workload is the
-LiDAR-like sweep: N = 1,000,000 points, C = 128 fp32 features, 0.2 m voxels.
+outside the timed region, ``test/test_scatter.py:24,38-44``).  The headline workload is
+the LiDAR-like sweep: N = 1,000,000 points, C = 128 fp32 features, 0.2 m voxels.
 Inputs are resident in HBM before the timed region starts.
 
 ``value`` is points per second per operator pass: ``2 * N / t_step`` (each step
@@ -15,9 +15,17 @@ durations are measured inside a second pass over the same steps, with a HIP even
 between the four entry-point calls; per-operator times, GB/s and roofline fractions
 derived from them are in ``per_kernel`` / ``per_op``.
 
+``other_configs`` holds the same measurements, GPU only and over fewer steps, for the
+other configurations: the uniform box, the half-precision sweep (fp16, bf16), the Zipf
+contention case, the four-sweep batch and the pillar binning of the sweep (the same
+points in 0.2 m x 0.2 m columns: the heavy-tailed occupancy, two thirds of the points in
+voxels that are split across wavefronts).
+
 Prints ONE JSON line on stdout.
 """
 import argparse
+import ctypes
+import hashlib
 import json
 import os
 import sys
@@ -30,17 +38,20 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-
-# HBM bytes per launch on the default workload (N=1,000,000, C=128, fp32), from two
-# rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by
-# what the same counter reads for the 512,000,000-byte device copy below (FETCH_SIZE
-# reads half of the copied bytes on this part: factor 2.000; WRITE_SIZE: factor 1.000).
-MEASURED_TRAFFIC_BYTES = {
-    "max_fwd": 525.4e6 + 334.7e6,
-    "max_bwd": 363.2e6 + 512.2e6,
-    "mean_fwd": 525.5e6 + 167.4e6,
-    "mean_bwd": 185.3e6 + 512.1e6,
-}
+TORCH_DTYPE = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+DTYPE_CODE = {"f32": 0, "f16": 1, "bf16": 2}
+OP_CODE = {"sum": 0, "mean": 1, "max": 2, "max_reftie": 3}
+WORKLOADS = ("lidar_sweep", "uniform_box", "zipf_contention", "multi_sweep", "reference_test_groups",
+             "lidar_pillars")
+# (workload, dtype) of the `other_configs` block, after the headline workload
+OTHER_CONFIGS = (("uniform_box", "f32"), ("lidar_sweep", "f16"), ("lidar_sweep", "bf16"),
+                 ("zipf_contention", "f32"), ("multi_sweep", "f32"), ("lidar_pillars", "f32"),
+                 ("lidar_pillars", "f16"))
+# HBM bytes per launch measured with rocprofv3 counters (FETCH_SIZE, WRITE_SIZE), per
+# (workload, dtype, kernel), together with a digest of the kernel sources they were
+# measured on: figures are reported only while the sources still match.
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_table.json")
+KERNEL_SOURCES = ("torchex_amd/csrc/scatter_kernels.hip", "torchex_amd/csrc/txs_common.h")
 
 
 def parse():
@@ -51,6 +62,9 @@ def parse():
     p.add_argument("--kernel-iters", type=int, default=50, help="launches per per-kernel timing loop")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-frontend", action="store_true", help="skip the front-end timings")
+    p.add_argument("--no-other-configs", action="store_true",
+                   help="measure the selected workload only (profiles of one workload use this)")
+    p.add_argument("--other-steps", type=int, default=12, help="timed steps per entry of other_configs")
     p.add_argument("--sorted-input", action="store_true",
                    help="also time the step on the same points delivered grouped by voxel "
                         "(off by default so that a profile of the default command holds one "
@@ -59,12 +73,10 @@ def parse():
                    help="also time each step kernel in a back-to-back loop of its own")
     p.add_argument("--points", type=int, default=1_000_000)
     p.add_argument("--channels", type=int, default=128)
-    p.add_argument("--workload", default="lidar_sweep",
-                   choices=("lidar_sweep", "uniform_box", "zipf_contention", "multi_sweep",
-                            "reference_test_groups"),
+    p.add_argument("--workload", default="lidar_sweep", choices=WORKLOADS,
                    help="lidar_sweep (default) is the workload the headline metric is quoted on; the "
                         "others run at their own fixed sizes and ignore --points/--channels")
-    p.add_argument("--dtype", default="f32", choices=("f32", "f16", "bf16"))
+    p.add_argument("--dtype", default="f32", choices=tuple(TORCH_DTYPE))
     return p.parse_args()
 
 
@@ -196,6 +208,145 @@ def frontend_timings(T, workloads, dev, N):
     return frontend
 
 
+class KernelNames:
+    """Asks the library which kernel instantiation it launches for given extents."""
+
+    def __init__(self):
+        from torchex_amd import _native
+        self.lib = _native.cabi()
+        self.lib.txs_kernel_name.restype = ctypes.c_int
+
+    def __call__(self, key, dtype, N, C, U):
+        op, direction = key.rsplit("_", 1)
+        buf = ctypes.create_string_buffer(64)
+        rc = self.lib.txs_kernel_name(ctypes.c_int(direction == "bwd"), ctypes.c_int(OP_CODE[op]),
+                                      ctypes.c_int(DTYPE_CODE[dtype]), ctypes.c_int64(N), ctypes.c_int64(C),
+                                      ctypes.c_int64(U), ctypes.c_int64(16), ctypes.c_int(1), buf,
+                                      ctypes.c_int64(64))
+        return buf.value.decode() if rc == 0 else None
+
+
+def load_traffic_table():
+    """Measured HBM bytes per launch, or {} with a note when the kernel sources have changed
+    since they were measured."""
+    if not os.path.exists(TRAFFIC_TABLE):
+        return {}, "no traffic table"
+    with open(TRAFFIC_TABLE) as f:
+        tab = json.load(f)
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    if h.hexdigest() != tab.get("kernel_sources_sha256"):
+        return {}, "kernel sources changed since the counters were collected (%s)" % tab.get("collected_with", "?")
+    return {(e["workload"], e["dtype"], e["kernel"]): e for e in tab["entries"]}, tab.get("collected_with")
+
+
+def make_workload(workloads, name, points, channels):
+    if name == "lidar_sweep":
+        return workloads.lidar_sweep(N=points, C=channels, seed=2)
+    return getattr(workloads, name)()
+
+
+def measure(T, scatter_ext, workloads, names, w, dtype, steps, warmup, dev, extras=False, kernel_iters=50):
+    """One workload at one dtype: the autograd step, then the step's four entry-point calls
+    timed one by one in step order."""
+    N, C, U = w.N, w.C, w.U
+    tdt = TORCH_DTYPE[dtype]
+    esz = 4 if dtype == "f32" else 2
+    g_mean_cpu = workloads.upstream_grad(U, C, 102)
+    g_max_cpu = workloads.upstream_grad(U, C, 103)
+    feats = w.feats.to(dev).to(tdt).requires_grad_(True)
+    inv, cnts = w.unq_inv.to(dev), w.unq_cnts.to(dev)
+    g_mean, g_max = g_mean_cpu.to(dev).to(tdt), g_max_cpu.to(dev).to(tdt)
+
+    data = T.ScatterData(inv, cnts)        # index preparation, timed separately
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        data = T.ScatterData(inv, cnts)
+    torch.cuda.synchronize()
+    prep_ms = (time.perf_counter() - t0) / 5 * 1e3
+
+    def step():
+        feats.grad = None
+        T.scatter_mean(feats, data).backward(g_mean)
+        feats.grad = None
+        mx, _ = T.scatter_max(feats, data)
+        mx.backward(g_max)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / steps * 1e3
+    feats.grad = None
+
+    # per-kernel durations inside the step: the same four entry-point calls in the same
+    # order as the timed region above, each bracketed by HIP events recorded on the
+    # stream the kernels are launched on (so every launch sees the cache state it sees
+    # in the step, not the one a back-to-back loop of one kernel leaves behind)
+    f = feats.detach()
+    plan = data.forward_args(C)
+    bplan = data.backward_args()
+    kt, kt_spread = instrumented_steps(scatter_ext, f, g_mean, g_max, plan, bplan, steps, warmup)
+    kernel_sum_ms = sum(kt.values())
+    res = {"N": N, "C": C, "U": U, "esz": esz, "data": data, "f": f, "g_mean": g_mean, "g_max": g_max,
+           "g_mean_cpu": g_mean_cpu, "g_max_cpu": g_max_cpu, "inv": inv, "cnts": cnts, "plan": plan,
+           "bplan": bplan, "prep_ms": prep_ms, "ms_per_step": ms_per_step, "kernel_sum_ms": kernel_sum_ms}
+    if extras:
+        # not part of the step: back-to-back launches of scatter_sum's kernels and of the
+        # forward under the reference's tie rule (what grouped input gets by default)
+        it = kernel_iters
+        kt["sum_fwd"] = event_ms(lambda: scatter_ext.forward(scatter_ext.SUM, f, *plan), it)
+        kt["sum_bwd"] = event_ms(lambda: scatter_ext.backward(scatter_ext.SUM, g_mean, None, *bplan), it)
+        kt["max_reftie_fwd"] = event_ms(lambda: scatter_ext.forward(scatter_ext.MAX_REFTIE, f, *plan), it)
+        res["max_fwd_back_to_back_ms"] = event_ms(lambda: scatter_ext.forward(scatter_ext.MAX, f, *plan), it)
+    ab = {k: workloads.algorithmic_bytes(k.replace("max_reftie", "max"), N, C, U, esz) for k in kt}
+    res["kt"] = kt
+    res["ab"] = ab
+    res["per_kernel"] = {k: {"kernel": names(k, dtype, N, C, U), "ms": kt[k], "GBps": ab[k] / kt[k] / 1e6,
+                             "frac": ab[k] / kt[k] / 1e6 / HBM_PEAK_GBPS, **kt_spread.get(k, {})}
+                         for k in kt}
+    per_op = {}
+    for op in ("mean", "max") + (("sum",) if extras else ()):
+        t = kt[op + "_fwd"] + kt[op + "_bwd"]
+        b = ab[op + "_fwd"] + ab[op + "_bwd"]
+        per_op[op] = {"ms_fwd": kt[op + "_fwd"], "ms_bwd": kt[op + "_bwd"], "points_per_s": N / t * 1e3,
+                      "GBps": b / t / 1e6, "frac_of_hbm_peak": b / t / 1e6 / HBM_PEAK_GBPS}
+    res["per_op"] = per_op
+    res["dominant"] = max(("max_fwd", "max_bwd", "mean_fwd", "mean_bwd"), key=lambda k: kt[k])
+    return res
+
+
+def workload_label(name, r, dtype):
+    d = r["data"]
+    return "%s N=%d C=%d %s, U=%d, max_cnt=%d, %s unq_inv%s" % (
+        name, r["N"], r["C"], dtype, r["U"], d.max_cnt, "sorted" if d.is_sorted else "unsorted",
+        ", voxel 0.2m" if name == "lidar_sweep" else ", pillar 0.2m x 0.2m" if name == "lidar_pillars" else "")
+
+
+def compact(name, dtype, r):
+    """The entry of one (workload, dtype) in other_configs."""
+    dom = r["dominant"]
+    step_bytes = sum(r["ab"][k] for k in ("mean_fwd", "mean_bwd", "max_fwd", "max_bwd"))
+    return {
+        "workload": workload_label(name, r, dtype), "dtype": dtype,
+        "U": r["U"], "max_cnt": r["data"].max_cnt, "num_heavy": r["data"].num_heavy,
+        "points_in_heavy_voxels": int(r["cnts"][r["cnts"] > r["data"].heavy_threshold].sum()),
+        "ms_per_step": r["ms_per_step"], "kernel_sum_ms": r["kernel_sum_ms"],
+        "points_per_s": 2 * r["N"] / r["ms_per_step"] * 1e3,
+        "step_frac_of_hbm_peak": step_bytes / r["kernel_sum_ms"] / 1e6 / HBM_PEAK_GBPS,
+        "per_op_frac": {op: v["frac_of_hbm_peak"] for op, v in r["per_op"].items()},
+        "per_kernel": {k: {"ms": v["ms"], "frac": v["frac"]} for k, v in r["per_kernel"].items()},
+        "dominant_kernel": r["per_kernel"][dom]["kernel"], "dominant_frac": r["per_kernel"][dom]["frac"],
+        "index_prep_ms": r["prep_ms"],
+    }
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -213,143 +364,103 @@ def main():
     from torchex_amd._native import scatter_ext
 
     dev = torch.device("cuda:0")
-    if a.workload == "lidar_sweep":
-        w = workloads.lidar_sweep(N=a.points, C=a.channels, seed=2)
-    else:
-        w = getattr(workloads, a.workload)()
-    N, C, U = w.N, w.C, w.U
-    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[a.dtype]
-    esz = 4 if a.dtype == "f32" else 2
-    g_mean_cpu = workloads.upstream_grad(U, C, 102)
-    g_max_cpu = workloads.upstream_grad(U, C, 103)
-
-    feats = w.feats.to(dev).to(tdt).requires_grad_(True)
-    inv, cnts = w.unq_inv.to(dev), w.unq_cnts.to(dev)
-    g_mean, g_max = g_mean_cpu.to(dev).to(tdt), g_max_cpu.to(dev).to(tdt)
-
-    # index preparation, timed separately
-    data = T.ScatterData(inv, cnts)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(5):
-        data = T.ScatterData(inv, cnts)
-    torch.cuda.synchronize()
-    prep_ms = (time.perf_counter() - t0) / 5 * 1e3
+    names = KernelNames()
+    w = make_workload(workloads, a.workload, a.points, a.channels)
+    r = measure(T, scatter_ext, workloads, names, w, a.dtype, a.steps, a.warmup, dev, extras=True,
+                kernel_iters=a.kernel_iters)
+    N, C, U, esz, data, f = r["N"], r["C"], r["U"], r["esz"], r["data"], r["f"]
+    kt, ab, per_kernel = r["kt"], r["ab"], r["per_kernel"]
+    scatter_fwd = scatter_ext.forward
 
     frontend = None
     if a.workload == "lidar_sweep" and not a.no_frontend:
         frontend = frontend_timings(T, workloads, dev, N)
 
-    def step():
-        feats.grad = None
-        T.scatter_mean(feats, data).backward(g_mean)
-        feats.grad = None
-        mx, _ = T.scatter_max(feats, data)
-        mx.backward(g_max)
-
-    for _ in range(a.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(a.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) / a.steps * 1e3
-
-    # per-kernel durations inside the step: the same four entry-point calls in the same
-    # order as the timed region above, each bracketed by HIP events recorded on the
-    # stream the kernels are launched on (so every launch sees the cache state it sees
-    # in the step, not the one a back-to-back loop of one kernel leaves behind)
-    f = feats.detach()
-    sc = data.scratch(C)
-    plan = (data.perm, data.seg, data.preSum, data.slot_of, data.heavy_ids, sc, data.max_cnt)
-    bplan = (data.perm, data.seg, data.preSum, N)
-    _, arg = scatter_ext.forward(scatter_ext.MAX, f, *plan)
-    kt, kt_spread = instrumented_steps(scatter_ext, f, g_mean, g_max, plan, bplan, a.steps, a.warmup)
-    kernel_sum_ms = sum(kt.values())
-
     # the same points delivered grouped by voxel, which is the only order the reference's
     # kernels accept (its getPreSum needs sorted ids): no row permutation, sequential writes
     sorted_input = None
     if a.sorted_input and not data.is_sorted:
-        order = torch.sort(inv, stable=True)[1]
+        order = torch.sort(r["inv"], stable=True)[1]
         f_s = f[order].contiguous()
-        data_s = T.ScatterData(inv[order].contiguous(), cnts)
-        plan_s = (data_s.perm, data_s.seg, data_s.preSum, data_s.slot_of, data_s.heavy_ids,
-                  data_s.scratch(C), data_s.max_cnt)
-        kts, _ = instrumented_steps(scatter_ext, f_s, g_mean, g_max, plan_s,
-                                    (data_s.perm, data_s.seg, data_s.preSum, N), a.steps, a.warmup)
+        data_s = T.ScatterData(r["inv"][order].contiguous(), r["cnts"])
+        plan_s = data_s.forward_args(C)
+        kts, _ = instrumented_steps(scatter_ext, f_s, r["g_mean"], r["g_max"], plan_s,
+                                    data_s.backward_args(), a.steps, a.warmup)
         sorted_input = {"per_kernel_ms": kts, "kernel_sum_ms": sum(kts.values()),
-                        "points_per_s": 2 * N / sum(kts.values()) * 1e3}
+                        "points_per_s": 2 * N / sum(kts.values()) * 1e3,
+                        "max_reftie_fwd_ms": event_ms(lambda: scatter_fwd(scatter_ext.MAX_REFTIE, f_s, *plan_s),
+                                                      a.kernel_iters)}
         del f_s, data_s, plan_s, order
 
-    # scatter_sum is not part of the step: back-to-back launches of its own kernels
-    it = a.kernel_iters
-    kt["sum_fwd"] = event_ms(lambda: scatter_ext.forward(scatter_ext.SUM, f, *plan), it)
-    kt["sum_bwd"] = event_ms(lambda: scatter_ext.backward(scatter_ext.SUM, g_mean, None, *bplan), it)
     isolated = None
     if a.isolated:
         # back-to-back launches of one entry point: upstream rows stay in the 256 MB
         # memory-side cache between launches, so the backward kernels read faster here
+        it, plan, bplan = a.kernel_iters, r["plan"], r["bplan"]
+        _, arg = scatter_fwd(scatter_ext.MAX, f, *plan)
         isolated = {
-            "mean_fwd": event_ms(lambda: scatter_ext.forward(scatter_ext.MEAN, f, *plan), it),
-            "mean_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MEAN, g_mean, None, *bplan), it),
-            "max_fwd": event_ms(lambda: scatter_ext.forward(scatter_ext.MAX, f, *plan), it),
-            "max_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MAX, g_max, arg, *bplan), it),
+            "mean_fwd": event_ms(lambda: scatter_fwd(scatter_ext.MEAN, f, *plan), it),
+            "mean_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MEAN, r["g_mean"], None, *bplan), it),
+            "max_fwd": event_ms(lambda: scatter_fwd(scatter_ext.MAX, f, *plan), it),
+            "max_bwd": event_ms(lambda: scatter_ext.backward(scatter_ext.MAX, r["g_max"], arg, *bplan), it),
         }
-    ab = {k: workloads.algorithmic_bytes(k, N, C, U, esz) for k in kt}
-    per_kernel = {k: {"ms": kt[k], "GBps": ab[k] / kt[k] / 1e6, "frac": ab[k] / kt[k] / 1e6 / HBM_PEAK_GBPS,
-                      **kt_spread.get(k, {})}
-                  for k in kt}
-    per_op = {}
-    for op in ("mean", "max", "sum"):
-        t = kt[op + "_fwd"] + kt[op + "_bwd"]
-        b = ab[op + "_fwd"] + ab[op + "_bwd"]
-        per_op[op] = {"ms_fwd": kt[op + "_fwd"], "ms_bwd": kt[op + "_bwd"], "points_per_s": N / t * 1e3,
-                      "GBps": b / t / 1e6, "frac_of_hbm_peak": b / t / 1e6 / HBM_PEAK_GBPS}
 
     # a plain device copy of the feature matrix on the same box: the practical ceiling
     dst = torch.empty_like(f)
     copy_ms = event_ms(lambda: dst.copy_(f), 20)
     copy_gbps = 2 * f.numel() * esz / copy_ms / 1e6
+    del dst
 
-    dom = max(("max_fwd", "max_bwd", "mean_fwd", "mean_bwd"), key=lambda k: kt[k])
-    row_bytes = C * esz
-    # elements per lane: 16-byte vectors for fp32, 8-byte ones for the 2-byte types
-    vec = next(v for v in ((16, 8, 4) if esz == 4 else (8, 4, 2)) if row_bytes % v == 0) // esz
-    kname = "scatter_%s_kernel<%s,%d,%s>" % (dom[-3:], a.dtype.upper(), vec, dom[:-4].upper())
-    if dom.endswith("bwd"):   # the backward kernel also carries its chunk (positions per lane group)
-        kname = kname[:-1] + (",8>" if N < 16 * U else ",16>")
-    roofline = {"bound": "hbm", "kernel": kname, "achieved": per_kernel[dom]["GBps"], "peak": HBM_PEAK_GBPS,
-                "unit": "GB/s", "frac": per_kernel[dom]["frac"],
-                "traffic": MEASURED_TRAFFIC_BYTES[dom]
-                if (a.workload, N, C, a.dtype) == ("lidar_sweep", 1_000_000, 128, "f32") else None,
+    dom = r["dominant"]
+    traffic_table, traffic_source = load_traffic_table()
+    entry = traffic_table.get((a.workload, a.dtype, per_kernel[dom]["kernel"]))
+    if a.workload == "lidar_sweep" and (N, C) != (1_000_000, 128):
+        entry = None    # the table holds the workloads at their default sizes
+    roofline = {"bound": "hbm", "kernel": per_kernel[dom]["kernel"], "achieved": per_kernel[dom]["GBps"],
+                "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": per_kernel[dom]["frac"],
+                "traffic": (entry["fetch_bytes"] + entry["write_bytes"]) if entry else None,
+                "traffic_source": (entry or {}).get("profile", traffic_source),
                 "algorithmic_bytes": ab[dom], "launch_ms": kt[dom]}
 
     out = {
         "metric": "scatter_mean+scatter_max(+argmax) fwd+bwd points/s (per operator pass), 1 GPU",
-        "value": 2 * N / ms_per_step * 1e3,
+        "value": 2 * N / r["ms_per_step"] * 1e3,
         "unit": "points/s",
-        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": r["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": a.dtype, "data": "synthetic",
-        "config": {"workload": "%s N=%d C=%d %s, U=%d, max_cnt=%d, %s unq_inv%s"
-                               % (a.workload, N, C, a.dtype, U, data.max_cnt,
-                                  "sorted" if data.is_sorted else "unsorted",
-                                  ", voxel 0.2m" if a.workload == "lidar_sweep" else ""),
-                   "num_special_voxels": data.num_special, "heavy_threshold": data.heavy_threshold},
+        "config": {"workload": workload_label(a.workload, r, a.dtype),
+                   "num_special_voxels": data.num_special, "num_heavy_voxels": data.num_heavy,
+                   "heavy_threshold": data.heavy_threshold},
         "roofline": roofline,
-        "per_op": per_op,
+        "per_op": r["per_op"],
         "per_kernel": per_kernel,
-        "kernel_sum_ms": kernel_sum_ms,
+        "kernel_sum_ms": r["kernel_sum_ms"],
+        "max_fwd_back_to_back_ms": r["max_fwd_back_to_back_ms"],
         "sorted_input": sorted_input,
         "device_copy_GBps": copy_gbps,
-        "index_prep_ms": prep_ms,
-        "step_incl_index_prep_ms": ms_per_step + prep_ms,
+        "index_prep_ms": r["prep_ms"],
+        "step_incl_index_prep_ms": r["ms_per_step"] + r["prep_ms"],
         "frontend": frontend,
     }
     if isolated is not None:
         out["per_kernel_isolated_ms"] = isolated
+    g_mean_cpu, g_max_cpu = r["g_mean_cpu"], r["g_max_cpu"]
+    del r, f, data
+    torch.cuda.empty_cache()
+
+    if not a.no_other_configs:
+        others = []
+        for name, dt in OTHER_CONFIGS:
+            if (name, dt) == (a.workload, a.dtype):
+                continue
+            wo = w if name == a.workload else make_workload(workloads, name, 1_000_000, 128)
+            ro = measure(T, scatter_ext, workloads, names, wo, dt, a.other_steps, 3, dev)
+            others.append(compact(name, dt, ro))
+            del ro, wo
+            torch.cuda.empty_cache()
+        out["other_configs"] = others
+
     if not a.no_cpu_baseline and a.dtype == "f32":
         out["cpu_baseline"] = cpu_baseline(w, g_mean_cpu, g_max_cpu)
     print(json.dumps(out), flush=True)

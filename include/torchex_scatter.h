@@ -26,10 +26,21 @@
  *                       in heavy_ids and its row in scratch), else -1
  *   heavy_ids  [n_special] int32 ids of the special voxels, the n_heavy heavy
  *                       ones first (slot order), the empty ones after them
- *   scratch    [n_heavy * C] 8-byte cells, one row per heavy voxel.  MUST BE
- *                       ZERO ON ENTRY to txs_scatter_forward and is zero again
- *                       when the call's kernels have finished.
+ *   scratch    8-byte cells: first [n_heavy * C], one row per heavy voxel, which
+ *                       MUST BE ZERO ON ENTRY to txs_scatter_forward and are zero again
+ *                       when the call's kernels have finished; behind them, room for
+ *                       the partial tables of table mode (never read before written,
+ *                       left dirty).  txs_scatter_scratch_cells() gives the total.
  *   out        [U, C]   dtype of feats;  arg [U, C] int32 (row index into feats)
+ *
+ * Table mode: when there are few voxels with many rows each (at least 512 rows per
+ * voxel on average) and a whole [U, C] table fits in the LDS of a compute unit, forward
+ * and backward run in ROW order instead of voxel order: the forward reduces contiguous
+ * spans of rows into per-workgroup LDS tables (LDS atomics), stores them as partial
+ * tables in `scratch` and combines them in a second kernel; the backward stages the
+ * upstream rows in LDS and writes the input gradient sequentially.  Rows narrower than
+ * a cache line are then read and written as a stream instead of one by one.  Table mode
+ * needs the row-order ids (unq_inv, or grouped rows) and, forward, the extra scratch.
  *
  * Special voxels: a voxel with more than `heavy_threshold` rows is reduced by
  * many wavefronts whose partials meet in `scratch` through atomics (fp32
@@ -56,6 +67,10 @@ enum {
 };
 enum { TXS_F32 = 0, TXS_F16 = 1, TXS_BF16 = 2 };
 enum { TXS_SUM = 0, TXS_MEAN = 1, TXS_MAX = 2, TXS_MAX_REFTIE = 3 };
+/* Which kernels a forward / backward call may use: the library's choice, the voxel-order
+ * kernels only, or the row-order table kernels only (TXS_ERR_UNSUPPORTED if they do not
+ * apply to the call). */
+enum { TXS_PATH_AUTO = 0, TXS_PATH_VOXEL_ORDER = 1, TXS_PATH_TABLE = 2 };
 
 /* Slots of the int32[TXS_STATS_LEN] device array the plan functions fill. */
 enum {
@@ -70,11 +85,23 @@ enum {
     TXS_STATS_LEN = 8
 };
 
-/* Library ABI version (7); bumped when a signature or the meaning of an argument changes. */
+/* Library ABI version (8); bumped when a signature or the meaning of an argument changes. */
 int txs_abi_version(void);
 
 /* Human-readable text for a status code. */
 const char *txs_status_string(int status);
+
+/* Name of the kernel instantiation that txs_scatter_forward (backward == 0) or
+ * txs_scatter_backward (backward != 0) launches for these extents, as a profiler lists
+ * it without namespaces ("scatter_fwd_kernel<F32,4,MAX>": dtype, elements per lane,
+ * operator; the backward kernel also carries its chunk length).  pointer_alignment is
+ * the alignment in bytes of the least aligned tensor (16 for ordinary allocations);
+ * table_allowed != 0 means the call would be made with TXS_PATH_AUTO, row-order ids and
+ * enough scratch ("table_fwd_kernel<F32,4,MAX>" is then reported where table mode applies).
+ * For logs and benchmarks; buf needs at least 48 bytes. */
+int txs_kernel_name(int backward, int op, int dtype, int64_t num_total, int64_t channel,
+                    int64_t num_unq, int64_t pointer_alignment, int table_allowed, char *buf,
+                    int64_t buf_len);
 
 /* Default population above which a voxel is reduced through atomics, and the
  * number of sorted positions one lane group walks. */
@@ -226,22 +253,33 @@ int txs_grid_hash_probe(const int32_t *keys, int64_t num_keys, const int32_t *ta
  *     -inf never wins, as in the reference.  max_cnt is the largest voxel
  *     population (the reference launcher's argument); other ops ignore it.
  * out (and arg) need no initialisation: every element is written.
- * scratch may be NULL when there is no heavy voxel (empty voxels need none). */
-int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *perm,
-                        const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
-                        const int32_t *heavy_ids, int64_t num_special, void *scratch,
-                        void *out, int32_t *arg, int64_t num_total, int64_t channel,
-                        int64_t num_unq, int64_t max_cnt, void *stream);
+ * unq_inv (may be NULL): the row-order voxel ids; without them (and with a perm)
+ *   table mode is not available.  num_heavy: TXS_STAT_NUM_HEAVY of the plan.
+ * scratch / scratch_cells: see "Data layout"; scratch may be NULL (scratch_cells 0) when
+ *   there is no heavy voxel.  With fewer than txs_scatter_scratch_cells() cells (but at
+ *   least num_heavy * channel) the call still works, on the voxel-order kernels.
+ * path: TXS_PATH_AUTO, or one of the other two to force a choice. */
+int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *unq_inv,
+                        const int32_t *perm, const int32_t *seg, const int32_t *preSum,
+                        const int32_t *slot_of, const int32_t *heavy_ids, int64_t num_special,
+                        int64_t num_heavy, void *scratch, int64_t scratch_cells, void *out,
+                        int32_t *arg, int64_t num_total, int64_t channel, int64_t num_unq,
+                        int64_t max_cnt, int path, void *stream);
+
+/* Number of 8-byte scratch cells that lets txs_scatter_forward choose freely between its
+ * kernels for these extents: num_heavy * channel, plus the partial tables of table mode
+ * where it applies.  -1 for invalid extents. */
+int64_t txs_scatter_scratch_cells(int64_t num_total, int64_t channel, int64_t num_unq,
+                                  int64_t num_heavy);
 
 /* txs_scatter_forward for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  Same arguments and results as txs_scatter_forward,
- * except that the heavy-voxel table is not passed in: the call uses a table that
- * lives in the library's own device image (one copy per GPU, 8 MiB, held until the
- * process ends), and num_heavy (TXS_STAT_NUM_HEAVY of the plan) says how many rows of
- * it are needed.  The call allocates and frees nothing and only launches kernels: it
- * clears the num_heavy * channel cells it is going to use, then runs the same kernels
- * as txs_scatter_forward.
+ * except that no scratch is passed in: the call uses a table that lives in the
+ * library's own device image (one copy per GPU, 8 MiB, held until the process ends).
+ * The call allocates and frees nothing and only launches kernels: it clears the
+ * num_heavy * channel cells the heavy voxels use, then runs the same kernels as
+ * txs_scatter_forward (table mode only where its partial tables fit in the rest).
  *   Limit: num_heavy * channel <= txs_resident_table_cells() (1,048,576 cells, e.g.
  *   8192 heavy voxels of 128 channels); beyond it the call returns TXS_ERR_TOO_LARGE
  *   and launches nothing.
@@ -251,11 +289,12 @@ int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *per
  *   The device that owns `stream` must be current.  The table's address is looked up
  *   the first time the call runs on a GPU; txs_resident_table_init() does that lookup
  *   ahead of time for the current GPU (call it before a graph capture starts). */
-int txs_scatter_forward_resident(int op, int dtype, const void *feats, const int32_t *perm,
-                                 const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
-                                 const int32_t *heavy_ids, int64_t num_special, int64_t num_heavy,
-                                 void *out, int32_t *arg, int64_t num_total, int64_t channel,
-                                 int64_t num_unq, int64_t max_cnt, void *stream);
+int txs_scatter_forward_resident(int op, int dtype, const void *feats, const int32_t *unq_inv,
+                                 const int32_t *perm, const int32_t *seg, const int32_t *preSum,
+                                 const int32_t *slot_of, const int32_t *heavy_ids, int64_t num_special,
+                                 int64_t num_heavy, void *out, int32_t *arg, int64_t num_total,
+                                 int64_t channel, int64_t num_unq, int64_t max_cnt, int path,
+                                 void *stream);
 int txs_resident_table_init(void);
 int64_t txs_resident_table_cells(void);
 
@@ -264,11 +303,12 @@ int64_t txs_resident_table_cells(void);
  * ScatterMeanFunction.backward (:74-78: (g / unq_cnts)[unq_inv]) and the
  * intended ScatterMaxFunction.backward (:106-111: zeros.scatter_(0, arg, g),
  * i.e. g_in[i,c] = g[u,c] if arg[u,c] == i else 0).
- * g_in [N, C] needs no initialisation.  arg is read only for TXS_MAX. */
+ * g_in [N, C] needs no initialisation.  arg is read only for TXS_MAX.
+ * unq_inv (may be NULL) and path: as for txs_scatter_forward. */
 int txs_scatter_backward(int op, int dtype, const void *grad_out, const int32_t *arg,
-                         const int32_t *perm, const int32_t *seg, const int32_t *preSum,
-                         void *grad_in, int64_t num_total, int64_t channel, int64_t num_unq,
-                         void *stream);
+                         const int32_t *unq_inv, const int32_t *perm, const int32_t *seg,
+                         const int32_t *preSum, void *grad_in, int64_t num_total, int64_t channel,
+                         int64_t num_unq, int path, void *stream);
 
 #ifdef __cplusplus
 }

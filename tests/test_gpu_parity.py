@@ -44,7 +44,7 @@ def bits_equal(a, b):
 
 
 def run_case(name, feats, unq_inv, unq_cnts, dtype=torch.float32, grad_seed=100, check_plan=True,
-             heavy_threshold=None, max_tie_rule=None):
+             heavy_threshold=None, max_tie_rule=None, path=None):
     """feats fp32 CPU [N, C]; unq_inv int64 CPU; unq_cnts int64 CPU.  Returns the
     ScatterData for extra checks.  scatter_max is checked against the oracle of the tie
     rule in force: by default the reference kernel's own winner (lane-exact emulation)
@@ -61,6 +61,8 @@ def run_case(name, feats, unq_inv, unq_cnts, dtype=torch.float32, grad_seed=100,
     fg = f_in.to(DEV).requires_grad_(True)
     data = T.ScatterData(unq_inv.to(DEV), unq_cnts.to(DEV), heavy_threshold=heavy_threshold,
                          max_tie_rule=max_tie_rule)
+    if path is not None:
+        data.path = path
     grouped = N < 2 or bool((unq_inv[1:] >= unq_inv[:-1]).all())
     assert data.is_sorted == grouped
     assert data.max_tie_rule == (max_tie_rule or ("reference" if grouped else "first"))
@@ -491,16 +493,20 @@ def test_c_abi_direct_call():
     f = feats.to(DEV)
     out = torch.empty((U, C), device=DEV)
     arg = torch.empty((U, C), device=DEV, dtype=torch.int32)
-    scratch = torch.zeros((max(data.num_special, 1) * C,), device=DEV, dtype=torch.int64)
+    lib.txs_scatter_scratch_cells.restype = ctypes.c_int64
     vp = ctypes.c_void_p
     i64 = ctypes.c_int64
+    cells = lib.txs_scatter_scratch_cells(i64(N), i64(C), i64(U), i64(data.num_heavy))
+    assert cells == data.num_heavy * C      # 300 voxels of ~17 rows: no table mode, no partial tables
+    scratch = torch.zeros((max(cells, 1),), device=DEV, dtype=torch.int64)
     stream = vp(torch.cuda.current_stream().cuda_stream)
     lib.txs_scatter_forward.restype = ctypes.c_int
     rc = lib.txs_scatter_forward(
-        ctypes.c_int(2), ctypes.c_int(0), vp(f.data_ptr()), vp(data.perm.data_ptr()), vp(data.seg.data_ptr()),
-        vp(data.preSum.data_ptr()), vp(data.slot_of.data_ptr()),
-        vp(data.heavy_ids.data_ptr() if data.num_special else 0), i64(data.num_special), vp(scratch.data_ptr()),
-        vp(out.data_ptr()), vp(arg.data_ptr()), i64(N), i64(C), i64(U), i64(data.max_cnt), stream)
+        ctypes.c_int(2), ctypes.c_int(0), vp(f.data_ptr()), vp(data.row_ids.data_ptr()), vp(data.perm.data_ptr()),
+        vp(data.seg.data_ptr()), vp(data.preSum.data_ptr()), vp(data.slot_of.data_ptr()),
+        vp(data.heavy_ids.data_ptr() if data.num_special else 0), i64(data.num_special), i64(data.num_heavy),
+        vp(scratch.data_ptr()), i64(cells), vp(out.data_ptr()), vp(arg.data_ptr()), i64(N), i64(C), i64(U),
+        i64(data.max_cnt), ctypes.c_int(0), stream)
     assert rc == 0
     torch.cuda.synchronize()
     wm, wa = orc.scatter_max_first(feats.numpy(), inv.numpy().astype(np.int32), U)
@@ -510,19 +516,20 @@ def test_c_abi_direct_call():
     gup = torch.randn((U, C), generator=g).to(DEV)
     lib.txs_scatter_backward.restype = ctypes.c_int
     rc = lib.txs_scatter_backward(
-        ctypes.c_int(2), ctypes.c_int(0), vp(gup.data_ptr()), vp(arg.data_ptr()), vp(data.perm.data_ptr()),
-        vp(data.seg.data_ptr()), vp(data.preSum.data_ptr()), vp(gin.data_ptr()), i64(N), i64(C), i64(U), stream)
+        ctypes.c_int(2), ctypes.c_int(0), vp(gup.data_ptr()), vp(arg.data_ptr()), vp(data.row_ids.data_ptr()),
+        vp(data.perm.data_ptr()), vp(data.seg.data_ptr()), vp(data.preSum.data_ptr()), vp(gin.data_ptr()),
+        i64(N), i64(C), i64(U), ctypes.c_int(0), stream)
     assert rc == 0
     torch.cuda.synchronize()
     assert bits_equal(gin.cpu().numpy(), orc.max_backward(gup.cpu().numpy(), wa, N))
     # argument validation returns a status instead of launching
     rc = lib.txs_scatter_forward(
-        ctypes.c_int(7), ctypes.c_int(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0), vp(0),
-        i64(N), i64(C), i64(U), i64(1), stream)
+        ctypes.c_int(7), ctypes.c_int(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), i64(0), vp(0),
+        i64(0), vp(0), vp(0), i64(N), i64(C), i64(U), i64(1), ctypes.c_int(0), stream)
     assert rc == 3
     rc = lib.txs_scatter_forward(
-        ctypes.c_int(0), ctypes.c_int(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0), vp(0),
-        i64(N), i64(C), i64(U), i64(1), stream)
+        ctypes.c_int(0), ctypes.c_int(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), i64(0), vp(0),
+        i64(0), vp(0), vp(0), i64(N), i64(C), i64(U), i64(1), ctypes.c_int(0), stream)
     assert rc == 1
 
 
@@ -667,7 +674,7 @@ def test_misaligned_views_fall_back_to_narrow_vectors():
         gbase = torch.empty(U * C + 3, device=DEV)
         gup = gbase[off:off + U * C].view(U, C)
         gup.copy_(workloads.upstream_grad(U, C, 5))
-        gin = scatter_ext.backward(scatter_ext.MAX, gup, arg, data.perm, data.seg, data.preSum, N)
+        gin = scatter_ext.backward(scatter_ext.MAX, gup, arg, *data.backward_args())
         assert bits_equal(gin.cpu().numpy(), orc.max_backward(gup.cpu().numpy(), wa, N))
 
 
@@ -704,8 +711,8 @@ def test_hip_graph_capture_and_replay():
         f = wl.feats.to(DEV)
         g = workloads.upstream_grad(U, C, 9).to(DEV)
         data = tx().ScatterData(inv, cnts)
-        plan = (data.perm, data.seg, data.preSum, data.slot_of, data.heavy_ids, data.scratch(C), data.max_cnt)
-        bplan = (data.perm, data.seg, data.preSum, N)
+        plan = data.forward_args(C)
+        bplan = data.backward_args()
 
         def run():
             mean, _ = scatter_ext.forward(scatter_ext.MEAN, f, *plan)
@@ -806,7 +813,7 @@ def test_mostly_empty_voxel_grid():
     feats = torch.randn((N, C), generator=g)
     data = run_case("mostly_empty", feats, inv, cnts)
     assert data.num_heavy == 1 and data.num_special == int((cnts == 0).sum()) + 1
-    assert tuple(data.scratch(C).shape) == (1, C)
+    assert tuple(data.scratch(C).shape) == (C,)
     # layout the kernels rely on: heavy voxels first, then the empty ones
     ids = data.heavy_ids.cpu()
     assert ids[0].item() == 123_456 and bool((cnts[ids[1:].long()] == 0).all())
@@ -973,11 +980,13 @@ def test_concurrent_streams_do_not_share_a_heavy_voxel_table():
     """Forwards of one ScatterData queued on two streams at the same time: each stream gets a
     heavy-voxel table of its own, so the results equal the single-stream ones."""
     T = tx()
+    from torchex_amd._native import scatter_ext
     w = workloads.zipf_contention(N=400_000, C=32, num_ids=300, seed=5)     # every voxel heavy
     inv, cnts = w.unq_inv.to(DEV), w.unq_cnts.to(DEV)
     fa = w.feats.to(DEV)
     fb = (w.feats * 0.5 + 1.0).to(DEV)
     data = T.ScatterData(inv, cnts)
+    data.path = scatter_ext.PATH_VOXEL_ORDER     # the kernels that merge heavy voxels through the table
     assert data.num_heavy == w.U
     ref_a, ref_b = T.scatter_max(fa, data), T.scatter_max(fb, data)
     torch.cuda.synchronize()
@@ -994,3 +1003,104 @@ def test_concurrent_streams_do_not_share_a_heavy_voxel_table():
     for mx, arg in outs_b:
         assert torch.equal(mx, ref_b[0]) and torch.equal(arg, ref_b[1])
     assert len(data._scratch) == 3 and all(not bool((t != 0).any()) for t in data._scratch.values())
+
+
+# ------------------------------------------------ few voxels: the row-order kernels --
+
+def _kernel_of(data, feats, backward, op):
+    from torchex_amd._native import scatter_ext
+    return scatter_ext.kernel_name(backward, op, feats, data.num_total, data.num_unq, True)
+
+
+def test_zipf_contention_takes_the_table_kernels_and_both_paths_agree():
+    """The contention workload (1024 voxels, 64-byte rows) is reduced in row order through
+    per-workgroup LDS tables; forcing the voxel-order kernels on the same plan gives the same
+    max / arg / gradients bit for bit and sums within tolerance."""
+    from torchex_amd._native import scatter_ext
+    T = tx()
+    w = workloads.zipf_contention()
+    f = w.feats.to(DEV)
+    data = T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV))
+    assert _kernel_of(data, f, False, scatter_ext.MAX).startswith("table_fwd_kernel")
+    assert _kernel_of(data, f, True, scatter_ext.MAX).startswith("table_bwd_kernel")
+    g = workloads.upstream_grad(w.U, w.C, 3).to(DEV)
+    res = {}
+    for path in (scatter_ext.PATH_TABLE, scatter_ext.PATH_VOXEL_ORDER):
+        data.path = path
+        x = f.clone().requires_grad_(True)
+        mx, arg = T.scatter_max(x, data)
+        mx.backward(g)
+        gmax = x.grad.clone()
+        x.grad = None
+        mean = T.scatter_mean(x, data)
+        mean.backward(g)
+        res[path] = (mx.detach(), arg, gmax, mean.detach(), x.grad.clone(), T.scatter_sum(f, data))
+    a, b = res[scatter_ext.PATH_TABLE], res[scatter_ext.PATH_VOXEL_ORDER]
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) and torch.equal(a[2], b[2])
+    assert torch.equal(a[4], b[4])
+    sabs = torch.zeros((w.U, w.C), device=DEV).index_add_(0, w.unq_inv.to(DEV), f.abs())
+    assert bool(((a[5] - b[5]).abs() <= 2e-5 * sabs).all())
+    assert bool(((a[3] - b[3]).abs() <= 2e-5 * sabs / data.unq_cnts).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("C", [1, 3, 4, 16, 20, 64])
+def test_table_kernels_channel_widths_and_dtypes(C, dtype):
+    from torchex_amd._native import scatter_ext
+    g = torch.Generator().manual_seed(500 + C)
+    N, U = 40_000, 37
+    inv = torch.randint(0, U, (N,), generator=g)
+    inv[inv == 5] = 6                       # an empty voxel
+    inv[:3000] = 11                         # a crowded one
+    feats = torch.randn((N, C), generator=g)
+    feats[torch.rand((N, C), generator=g) < 0.1] = 0.5      # ties
+    run_case(f"table C={C}", feats, inv, torch.bincount(inv, minlength=U), dtype=dtype,
+             path=scatter_ext.PATH_TABLE)
+
+
+def test_table_kernels_special_values_and_grouped_rows():
+    from torchex_amd._native import scatter_ext
+    g = torch.Generator().manual_seed(9)
+    N, U, C = 30_000, 24, 8
+    inv = torch.randint(0, U, (N,), generator=g)
+    f = torch.randn((N, C), generator=g)
+    f[torch.rand((N, C), generator=g) < 0.05] = float("nan")
+    f[torch.rand((N, C), generator=g) < 0.05] = float("-inf")
+    f[torch.rand((N, C), generator=g) < 0.02] = float("inf")
+    f[torch.rand((N, C), generator=g) < 0.05] = -0.0
+    f[torch.rand((N, C), generator=g) < 0.05] = 0.0
+    f[inv == 0] = float("nan")
+    f[inv == 1] = float("-inf")
+    f[inv == 2] = -0.0
+    rows3 = torch.nonzero(inv == 3).flatten()
+    f[rows3] = -0.0
+    f[rows3[len(rows3) // 2:]] = 0.0        # first maximal row holds -0.0: its bits are the result
+    T = tx()
+    cnts = torch.bincount(inv, minlength=U)
+    for path in (scatter_ext.PATH_TABLE, scatter_ext.PATH_VOXEL_ORDER):
+        data = T.ScatterData(inv.to(DEV), cnts.to(DEV))
+        data.path = path
+        mx, arg = T.scatter_max(f.to(DEV), data)
+        wm, wa = orc.scatter_max_first(f.numpy(), inv.numpy().astype(np.int32), U)
+        assert np.array_equal(arg.cpu().numpy(), wa), path
+        assert bits_equal(mx.cpu().numpy(), wm), path
+        assert np.signbit(mx.cpu().numpy()[2]).all() and np.signbit(mx.cpu().numpy()[3]).all()
+        s = T.scatter_sum(f.to(DEV), data).cpu().numpy()
+        ws = orc.scatter_sum_f64(f.numpy(), inv.numpy().astype(np.int32), U)
+        assert np.array_equal(np.isnan(s), np.isnan(ws)) and np.array_equal(np.isinf(s), np.isinf(ws))
+    # grouped rows (no permutation): the first-row rule through the table kernels; the
+    # reference's tie rule needs voxel order and says so when the table kernels are forced
+    order = torch.argsort(inv, stable=True)
+    fin = torch.randint(-3, 4, (N, C), generator=g).float()
+    run_case("table grouped", fin[order], inv[order], cnts, max_tie_rule="first", path=scatter_ext.PATH_TABLE)
+    dref = T.ScatterData(inv[order].to(DEV), cnts.to(DEV))
+    assert dref.max_tie_rule == "reference"
+    dref.path = scatter_ext.PATH_TABLE
+    with pytest.raises(RuntimeError, match="unsupported"):
+        T.scatter_max(fin[order].to(DEV), dref)
+    # many voxels: the table kernels do not apply
+    w = workloads.lidar_sweep(N=50_000, C=16, seed=4)
+    dl = T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV))
+    dl.path = scatter_ext.PATH_TABLE
+    with pytest.raises(RuntimeError, match="unsupported"):
+        T.scatter_sum(w.feats.to(DEV), dl)

@@ -40,7 +40,7 @@ def test_header_is_plain_c_and_links(tmp_path):
         pytest.skip("no C compiler on this machine")
     src = tmp_path / "abi.c"
     src.write_text('#include "torchex_scatter.h"\n'
-                   'int main(void) { return txs_abi_version() == 7 && txs_chunk_rows() > 0 ? 0 : 1; }\n')
+                   'int main(void) { return txs_abi_version() == 8 && txs_chunk_rows() > 0 ? 0 : 1; }\n')
     inc = os.path.join(ROOT, "include")
     pkg = os.path.join(ROOT, "torchex_amd")
     subprocess.check_call([cc, "-std=c11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I" + inc,
@@ -53,7 +53,7 @@ def test_header_is_plain_c_and_links(tmp_path):
 
 def test_host_only_entry_points():
     lib = _lib()
-    assert lib.txs_abi_version() == 7
+    assert lib.txs_abi_version() == 8
     lib.txs_status_string.restype = ctypes.c_char_p
     assert lib.txs_status_string(0) == b"ok"
     assert b"invalid" in lib.txs_status_string(1)
@@ -68,18 +68,28 @@ def test_argument_validation_needs_no_gpu():
     # these return before any launch
     lib = _lib()
     vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
-    rc = lib.txs_scatter_forward(ci(9), ci(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0),
-                                 vp(0), i64(1), i64(1), i64(1), i64(1), vp(0))
-    assert rc == 3
-    rc = lib.txs_scatter_forward(ci(0), ci(5), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0),
-                                 vp(0), i64(1), i64(1), i64(1), i64(1), vp(0))
-    assert rc == 3
-    rc = lib.txs_scatter_forward(ci(0), ci(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0), vp(0), vp(0),
-                                 vp(0), i64(1 << 40), i64(1), i64(1), i64(1), vp(0))
+    def fwd(op, dtype, num_total, path=0):
+        return lib.txs_scatter_forward(ci(op), ci(dtype), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(0),
+                                       i64(0), vp(0), i64(0), vp(0), vp(0), i64(num_total), i64(1), i64(1), i64(1),
+                                       ci(path), vp(0))
+    assert fwd(9, 0, 1) == 3
+    assert fwd(0, 5, 1) == 3
+    assert fwd(0, 0, 1, path=7) == 3
+    assert fwd(0, 0, 1 << 40) == 1
+    rc = lib.txs_scatter_backward(ci(2), ci(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(5), i64(4),
+                                  i64(2), ci(0), vp(0))
     assert rc == 1
-    rc = lib.txs_scatter_backward(ci(2), ci(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), i64(5), i64(4), i64(2),
-                                  vp(0))
-    assert rc == 1
+    # scratch sizing and kernel naming are host-only too
+    lib.txs_scatter_scratch_cells.restype = ctypes.c_int64
+    assert lib.txs_scatter_scratch_cells(i64(1_000_000), i64(128), i64(300_000), i64(10)) == 1280
+    assert lib.txs_scatter_scratch_cells(i64(-1), i64(128), i64(3), i64(0)) == -1
+    buf = ctypes.create_string_buffer(64)
+    assert lib.txs_kernel_name(ci(0), ci(2), ci(0), i64(1_000_000), i64(128), i64(300_000), i64(16), ci(1), buf,
+                               i64(64)) == 0
+    assert buf.value == b"scatter_fwd_kernel<F32,4,MAX>"
+    assert lib.txs_kernel_name(ci(1), ci(1), ci(1), i64(1_000_000), i64(128), i64(300_000), i64(16), ci(1), buf,
+                               i64(64)) == 0
+    assert buf.value == b"scatter_bwd_kernel<F16,4,MEAN,8>"
     rc = lib.txs_get_presum(vp(0), vp(0), i64(-1), i64(0), vp(0))
     assert rc == 1
 

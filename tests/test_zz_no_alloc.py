@@ -18,6 +18,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 SUM, MEAN, MAX = 0, 1, 2
 F32 = 0
+VOXEL_ORDER = 1    # both calls on the voxel-order kernels, the ones that use the heavy-voxel table
 
 
 def _say(*a):
@@ -33,17 +34,21 @@ def _forward(lib, resident, op, f, data, stream):
     arg = torch.full((U, C), -7, device=DEV, dtype=torch.int32)
     perm = vp(data.perm.data_ptr()) if data.perm is not None else vp(0)
     heavy = vp(data.heavy_ids.data_ptr() if data.num_special else 0)
-    common_head = (ci(op), ci(F32), vp(f.data_ptr()), perm, vp(data.seg.data_ptr()), vp(data.preSum.data_ptr()),
-                   vp(data.slot_of.data_ptr()), heavy, i64(data.num_special))
-    common_tail = (vp(out.data_ptr()), vp(arg.data_ptr()), i64(N), i64(C), i64(U), i64(data.max_cnt), stream)
+    ids = vp(data.row_ids.data_ptr()) if data.row_ids is not None else vp(0)
+    common_head = (ci(op), ci(F32), vp(f.data_ptr()), ids, perm, vp(data.seg.data_ptr()),
+                   vp(data.preSum.data_ptr()), vp(data.slot_of.data_ptr()), heavy, i64(data.num_special),
+                   i64(data.num_heavy))
+    common_tail = (vp(out.data_ptr()), vp(arg.data_ptr()), i64(N), i64(C), i64(U), i64(data.max_cnt),
+                   ci(VOXEL_ORDER), stream)
     if resident:
         lib.txs_scatter_forward_resident.restype = ctypes.c_int
-        rc = lib.txs_scatter_forward_resident(*common_head, i64(data.num_heavy), *common_tail)
+        rc = lib.txs_scatter_forward_resident(*common_head, *common_tail)
         table = None
     else:
-        table = torch.zeros((max(data.num_heavy, 1) * C,), device=DEV, dtype=torch.int64)
+        cells = max(data.num_heavy, 1) * C
+        table = torch.zeros((cells,), device=DEV, dtype=torch.int64)
         lib.txs_scatter_forward.restype = ctypes.c_int
-        rc = lib.txs_scatter_forward(*common_head, vp(table.data_ptr()), *common_tail)
+        rc = lib.txs_scatter_forward(*common_head, vp(table.data_ptr()), i64(cells), *common_tail)
     assert rc == 0, rc
     torch.cuda.synchronize()
     return out, arg
@@ -87,8 +92,8 @@ def test_resident_table_forward_matches_caller_table_forward():
     out = torch.full((wide.U, 8), 7.0, device=DEV)
     lib.txs_scatter_forward_resident.restype = ctypes.c_int
     rc = lib.txs_scatter_forward_resident(
-        ci(SUM), ci(F32), vp(1), vp(0), vp(1), vp(1), vp(1), vp(1), i64(2_000_000), i64(2_000_000),
-        vp(out.data_ptr()), vp(0), i64(10), i64(8), i64(2_000_000), i64(1), stream)
+        ci(SUM), ci(F32), vp(1), vp(0), vp(0), vp(1), vp(1), vp(1), vp(1), i64(2_000_000), i64(2_000_000),
+        vp(out.data_ptr()), vp(0), i64(10), i64(8), i64(2_000_000), i64(1), ci(0), stream)
     assert rc == 4
     lib.txs_status_string.restype = ctypes.c_char_p
     assert b"exceeds" in lib.txs_status_string(4)

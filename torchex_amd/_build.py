@@ -1,7 +1,7 @@
 """In-tree build of the two native pieces (run on a CPU-only machine; hipcc
 cross-compiles for gfx950):
 
-``libtorchex_scatter.so``  HIP kernels + C ABI (three translation units under
+``libtorchex_scatter.so``  HIP kernels + C ABI (four translation units under
                            ``csrc/``), built with hipcc, no torch in it.
 ``scatter_ext*.so``        the PyTorch C++ extension module, built with the host
                            compiler against the torch headers; links to the
@@ -29,7 +29,7 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
-KERNEL_SOURCES = ["plan_kernels.hip", "frontend_kernels.hip", "scatter_kernels.hip"]
+KERNEL_SOURCES = ["plan_kernels.hip", "frontend_kernels.hip", "scatter_kernels.hip", "table_kernels.hip"]
 OBJ_DIR = os.path.join(PKG, "_obj")
 
 

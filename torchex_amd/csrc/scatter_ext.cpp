@@ -314,22 +314,33 @@ Tensor grid_hash_probe(const Tensor &coors, const Tensor &table) {
     return out;
 }
 
-// one zeroed row of 8-byte cells per heavy voxel (empty voxels need none)
-Tensor make_scratch(int64_t num_heavy, int64_t C, const Tensor &like) {
-    return at::zeros({num_heavy, C}, like.options().dtype(at::kLong));
+// Zeroed scratch for forward calls on a [num_total, channel] feature matrix: the heavy
+// voxels' rows first (which the kernels leave zeroed), behind them room for the partial
+// tables of table mode where it applies.
+Tensor make_scratch(int64_t num_total, int64_t channel, int64_t num_unq, int64_t num_heavy, const Tensor &like) {
+    const int64_t cells = txs_scatter_scratch_cells(num_total, channel, num_unq, num_heavy);
+    TORCH_CHECK(cells >= 0, "make_scratch: invalid extents");
+    return at::zeros({cells}, like.options().dtype(at::kLong));
 }
 
-void run_forward(int op, const Tensor &feats, const OptTensor &perm, const Tensor &seg,
-                 const Tensor &preSum, const Tensor &slot_of, const Tensor &heavy_ids,
-                 Tensor &scratch, Tensor &out, OptTensor &arg, int64_t max_cnt) {
+int check_path(int64_t path) {
+    TORCH_CHECK(path == TXS_PATH_AUTO || path == TXS_PATH_VOXEL_ORDER || path == TXS_PATH_TABLE,
+                "path must be 0 (auto), 1 (voxel-order kernels) or 2 (table kernels)");
+    return (int)path;
+}
+
+void run_forward(int op, const Tensor &feats, const OptTensor &unq_inv, const OptTensor &perm, const Tensor &seg,
+                 const Tensor &preSum, const Tensor &slot_of, const Tensor &heavy_ids, int64_t num_heavy,
+                 Tensor &scratch, Tensor &out, OptTensor &arg, int64_t max_cnt, int path) {
     const int64_t N = feats.size(0), C = feats.size(1), U = preSum.numel() - 1;
     const int64_t S = heavy_ids.numel();
-    TORCH_CHECK(scratch.dim() == 2 && (scratch.size(0) == 0 || scratch.size(1) == C),
-                "scratch must be [num_heavy, channel] (ScatterData.scratch(channel))");
-    const int64_t H = scratch.size(0);
-    TORCH_CHECK(H <= S, "scratch has more rows than there are special voxels");
+    TORCH_CHECK(scratch.dim() == 1, "scratch must be 1-D (ScatterData.scratch(channel))");
+    TORCH_CHECK(num_heavy >= 0 && num_heavy <= S, "num_heavy exceeds the number of special voxels");
+    TORCH_CHECK(scratch.numel() >= num_heavy * C, "scratch holds ", scratch.numel(), " cells, the heavy voxels need ",
+                num_heavy * C);
     TORCH_CHECK(seg.numel() == N, "plan was built for ", seg.numel(), " rows, feats has ", N);
     TORCH_CHECK(!perm.has_value() || perm->numel() == N, "perm length mismatch");
+    TORCH_CHECK(!unq_inv.has_value() || unq_inv->numel() == N, "unq_inv length mismatch");
     TORCH_CHECK(slot_of.numel() == U, "slot_of length mismatch");
     TORCH_CHECK(out.size(0) == U && out.size(1) == C, "out must be [num_unq, channel]");
     const int dt = dtype_code(feats, "feats");
@@ -337,20 +348,21 @@ void run_forward(int op, const Tensor &feats, const OptTensor &perm, const Tenso
     int rc;
     {
         pybind11::gil_scoped_release nogil;
-        rc = txs_scatter_forward(op, dt, feats.data_ptr(), opt_i32p(perm), i32p(seg), i32p(preSum),
-                                 i32p(slot_of), i32p(heavy_ids), S,
-                                 H ? scratch.data_ptr() : nullptr, out.data_ptr(),
-                                 arg.has_value() ? arg->data_ptr<int32_t>() : nullptr, N, C, U, max_cnt,
+        rc = txs_scatter_forward(op, dt, feats.data_ptr(), opt_i32p(unq_inv), opt_i32p(perm), i32p(seg),
+                                 i32p(preSum), i32p(slot_of), i32p(heavy_ids), S, num_heavy,
+                                 scratch.numel() ? scratch.data_ptr() : nullptr, scratch.numel(), out.data_ptr(),
+                                 arg.has_value() ? arg->data_ptr<int32_t>() : nullptr, N, C, U, max_cnt, path,
                                  st);
     }
     check_status(rc, "scatter_forward");
 }
 
-// forward(op, feats, perm|None, seg, preSum, slot_of, heavy_ids, scratch, max_cnt) -> (out, arg|None)
-std::tuple<Tensor, OptTensor> forward(int64_t op, const Tensor &feats, const OptTensor &perm,
-                                      const Tensor &seg, const Tensor &preSum,
-                                      const Tensor &slot_of, const Tensor &heavy_ids,
-                                      Tensor scratch, int64_t max_cnt) {
+// forward(op, feats, unq_inv|None, perm|None, seg, preSum, slot_of, heavy_ids, num_heavy, scratch, max_cnt,
+//         path=0) -> (out, arg|None)
+std::tuple<Tensor, OptTensor> forward(int64_t op, const Tensor &feats, const OptTensor &unq_inv,
+                                      const OptTensor &perm, const Tensor &seg, const Tensor &preSum,
+                                      const Tensor &slot_of, const Tensor &heavy_ids, int64_t num_heavy,
+                                      Tensor scratch, int64_t max_cnt, int64_t path) {
     check_dev(feats, "feats");
     TORCH_CHECK(feats.dim() == 2, "feats must be [num_total, channel]");
     check_i32(seg, "seg");
@@ -358,6 +370,7 @@ std::tuple<Tensor, OptTensor> forward(int64_t op, const Tensor &feats, const Opt
     check_i32(slot_of, "slot_of");
     check_i32(heavy_ids, "heavy_ids");
     if (perm.has_value()) check_i32(*perm, "perm");
+    if (unq_inv.has_value()) check_i32(*unq_inv, "unq_inv");
     check_dev(scratch, "scratch");
     TORCH_CHECK(scratch.scalar_type() == at::kLong, "scratch must be int64");
     TORCH_CHECK(seg.device() == feats.device(), "plan and feats live on different devices");
@@ -366,22 +379,25 @@ std::tuple<Tensor, OptTensor> forward(int64_t op, const Tensor &feats, const Opt
     Tensor out = at::empty({U, C}, feats.options());
     OptTensor arg;
     if (op == TXS_MAX || op == TXS_MAX_REFTIE) arg = at::empty({U, C}, feats.options().dtype(at::kInt));
-    run_forward((int)op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, out, arg, max_cnt);
+    run_forward((int)op, feats, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_heavy, scratch, out, arg, max_cnt,
+                check_path(path));
     return {out, arg};
 }
 
-// backward(op, grad_out, arg|None, perm|None, seg, preSum, num_total) -> grad_in
-Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const OptTensor &perm,
-                const Tensor &seg, const Tensor &preSum, int64_t num_total) {
+// backward(op, grad_out, arg|None, unq_inv|None, perm|None, seg, preSum, num_total, path=0) -> grad_in
+Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const OptTensor &unq_inv,
+                const OptTensor &perm, const Tensor &seg, const Tensor &preSum, int64_t num_total, int64_t path) {
     check_dev(grad_out, "grad_out");
     TORCH_CHECK(grad_out.dim() == 2, "grad_out must be [num_unq, channel]");
     check_i32(seg, "seg");
     check_i32(preSum, "preSum");
     if (perm.has_value()) check_i32(*perm, "perm");
+    if (unq_inv.has_value()) check_i32(*unq_inv, "unq_inv");
     const int64_t U = preSum.numel() - 1, C = grad_out.size(1), N = num_total;
     TORCH_CHECK(grad_out.size(0) == U, "grad_out has ", grad_out.size(0), " rows, plan has ", U, " voxels");
     TORCH_CHECK(seg.numel() == N, "plan row count mismatch");
     TORCH_CHECK(!perm.has_value() || perm->numel() == N, "perm length mismatch");
+    TORCH_CHECK(!unq_inv.has_value() || unq_inv->numel() == N, "unq_inv length mismatch");
     TORCH_CHECK(seg.device() == grad_out.device(), "plan and grad_out live on different devices");
     if (op == TXS_MAX || op == TXS_MAX_REFTIE) {
         TORCH_CHECK(arg.has_value(), "scatter_max backward needs arg");
@@ -390,13 +406,14 @@ Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const 
     }
     c10::hip::HIPGuardMasqueradingAsCUDA guard(grad_out.device());
     const int dt = dtype_code(grad_out, "grad_out");
+    const int pth = check_path(path);
     Tensor gin = at::empty({N, C}, grad_out.options());
     void *st = cur_stream(grad_out);
     int rc;
     {
         pybind11::gil_scoped_release nogil;
-        rc = txs_scatter_backward((int)op, dt, grad_out.data_ptr(), opt_i32p(arg), opt_i32p(perm),
-                                  i32p(seg), i32p(preSum), gin.data_ptr(), N, C, U, st);
+        rc = txs_scatter_backward((int)op, dt, grad_out.data_ptr(), opt_i32p(arg), opt_i32p(unq_inv),
+                                  opt_i32p(perm), i32p(seg), i32p(preSum), gin.data_ptr(), N, C, U, pth, st);
     }
     check_status(rc, "scatter_backward");
     return gin;
@@ -492,20 +509,23 @@ void csr_reduce(int op, Tensor feats, Tensor preSum, Tensor out, OptTensor arg, 
     // value) while the GIL is held: run_forward releases it, and another Python thread
     // may then insert into or reorder the cache.
     Tensor seg, slot_of, heavy_ids, scratch;
+    int64_t num_heavy = 0;
     {
         CsrPlan &plan = csr_plan_for(preSum, feats.size(0));
         for (auto &entry : plan.scratch)
             if (std::get<0>(entry) == C && std::get<1>(entry) == st) scratch = std::get<2>(entry);
         if (!scratch.defined()) {
-            scratch = make_scratch(plan.num_heavy, C, feats);
+            scratch = make_scratch(feats.size(0), C, preSum.numel() - 1, plan.num_heavy, feats);
             plan.scratch.emplace_back(C, st, scratch);
         }
         seg = plan.seg;
         slot_of = plan.slot_of;
         heavy_ids = plan.heavy_ids;
+        num_heavy = plan.num_heavy;
     }
-    OptTensor perm;
-    run_forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, out, arg, max_cnt);
+    OptTensor perm, unq_inv;  // grouped rows: the per-position ids are the row-order ids
+    run_forward(op, feats, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_heavy, scratch, out, arg, max_cnt,
+                TXS_PATH_AUTO);
 }
 
 void clear_csr_plan_cache() { csr_plan_cache().clear(); }
@@ -559,11 +579,29 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("dynamic_point_pool", &dynamic_point_pool, "dynamic_point_pool(rois, pts, extra_wlh, max_pts_per_box, max_all_pts)");
     m.def("grid_hash_build", &grid_hash_build, "build_table(coors, values) -> table");
     m.def("grid_hash_probe", &grid_hash_probe, "probe_table(coors, table) -> values");
-    m.def("make_scratch", &make_scratch, "zeroed scratch table, one row per heavy voxel");
+    m.def("make_scratch", &make_scratch, "make_scratch(num_total, channel, num_unq, num_heavy, like): zeroed forward scratch");
     m.def("clear_csr_plan_cache", &clear_csr_plan_cache, "drop the plans kept for sum/max over CSR offsets");
     m.def("csr_plan_cache_size", &csr_plan_cache_size, "number of plans currently kept for sum/max over CSR offsets");
-    m.def("forward", &forward, "forward(op, feats, perm, seg, preSum, slot_of, heavy_ids, scratch, max_cnt)");
-    m.def("backward", &backward, "backward(op, grad_out, arg, perm, seg, preSum, num_total)");
+    m.def("forward", &forward,
+          "forward(op, feats, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_heavy, scratch, max_cnt, path=0)",
+          pybind11::arg("op"), pybind11::arg("feats"), pybind11::arg("unq_inv"), pybind11::arg("perm"),
+          pybind11::arg("seg"), pybind11::arg("preSum"), pybind11::arg("slot_of"), pybind11::arg("heavy_ids"),
+          pybind11::arg("num_heavy"), pybind11::arg("scratch"), pybind11::arg("max_cnt"), pybind11::arg("path") = 0);
+    m.def("backward", &backward, "backward(op, grad_out, arg, unq_inv, perm, seg, preSum, num_total, path=0)",
+          pybind11::arg("op"), pybind11::arg("grad_out"), pybind11::arg("arg"), pybind11::arg("unq_inv"),
+          pybind11::arg("perm"), pybind11::arg("seg"), pybind11::arg("preSum"), pybind11::arg("num_total"),
+          pybind11::arg("path") = 0);
+    m.def("kernel_name", [](bool backward, int64_t op, const Tensor &like, int64_t num_total, int64_t num_unq,
+                            bool table_allowed) {
+        char buf[64];
+        check_status(txs_kernel_name(backward, (int)op, dtype_code(like, "like"), num_total, like.size(1), num_unq, 16,
+                                     table_allowed, buf, 64),
+                     "kernel_name");
+        return std::string(buf);
+    }, "kernel_name(backward, op, like, num_total, num_unq, table_allowed): the kernel a call on `like`-shaped rows launches");
+    m.attr("PATH_AUTO") = (int)TXS_PATH_AUTO;
+    m.attr("PATH_VOXEL_ORDER") = (int)TXS_PATH_VOXEL_ORDER;
+    m.attr("PATH_TABLE") = (int)TXS_PATH_TABLE;
     m.def("abi_version", &txs_abi_version);
     m.def("default_heavy_threshold", &txs_default_heavy_threshold);
     m.attr("SUM") = (int)TXS_SUM;

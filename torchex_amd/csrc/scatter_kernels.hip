@@ -27,6 +27,9 @@
 
 #include "txs_common.h"
 
+#include <stdio.h>
+
+#include <initializer_list>
 #include <mutex>
 
 // Heavy-voxel table that lives in the library's own device image, for callers that cannot
@@ -84,6 +87,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     unsigned long long *__restrict__ scratch, const int *__restrict__ preSum, int N, int C, int U,
     int lpr_log2, int ref_log2) {
     using raw = typename TR::raw;
+    constexpr int kBatch = sizeof(raw) == 2 ? kBatchHalf : ::kBatch;
     constexpr bool kMax = OP == TXS_MAX || OP == TXS_MAX_REFTIE;
     constexpr bool kRef = OP == TXS_MAX_REFTIE;  // idx[] then holds ref_key, not a row
     extern __shared__ int lds[];
@@ -480,6 +484,7 @@ __global__ __launch_bounds__(kThreads) void scatter_bwd_kernel(
     const int *__restrict__ perm, const int *__restrict__ seg, const int *__restrict__ preSum,
     typename TR::raw *__restrict__ gin, int N, int C, int U, int lpr_log2) {
     using raw = typename TR::raw;
+    constexpr int kBatchBwd = sizeof(raw) == 2 ? kBatchBwdHalf : ::kBatchBwd;
     extern __shared__ int lds[];
     const int G = kThreads >> lpr_log2;
     const int T = G * CHUNK;
@@ -668,7 +673,7 @@ hipError_t launch_fwd(int op, const Geometry &geo, hipStream_t st, const void *f
     if (geo.vec_bytes == VB)                                                                     \
         return launch_fwd_op<TR, (VB) / e>(op, geo, st, feats, perm, seg, preSum, slot_of, out,  \
                                            arg, scratch, N, C, U, ref_log2);
-    if constexpr (e == 4) {
+    if constexpr (e == 4 || kHalfVecBytes == 16) {
         TXS_FWD(16)
     }
     TXS_FWD(8)
@@ -754,7 +759,7 @@ hipError_t launch_bwd(int op, const Geometry &geo, hipStream_t st, const void *g
 #define TXS_BWD(VB)                                                                               \
     if (geo.vec_bytes == VB)                                                                      \
         return launch_bwd_op<TR, (VB) / e>(op, geo, st, g, arg, perm, seg, preSum, gin, N, C, U);
-    if constexpr (e == 4) {
+    if constexpr (e == 4 || kHalfVecBytes == 16) {
         TXS_BWD(16)
     }
     TXS_BWD(8)
@@ -766,29 +771,60 @@ hipError_t launch_bwd(int op, const Geometry &geo, hipStream_t st, const void *g
     return hipErrorInvalidValue;
 }
 
-// Argument checks and the two launches (reduction, then the special voxels' rows) behind
-// txs_scatter_forward and txs_scatter_forward_resident.
-int scatter_forward_impl(int op, int dtype, const void *feats, const int32_t *perm,
+// Largest power of two (up to 16) that divides every given address.
+long common_alignment(std::initializer_list<const void *> ptrs) {
+    uintptr_t bits = 16;
+    for (const void *p : ptrs) bits |= (uintptr_t)p;
+    return (long)(bits & (~bits + 1));
+}
+
+// Row-order ids for the table kernels: unq_inv itself, or for grouped rows (no perm) the
+// per-position ids, whose bit 31 the kernels mask off.
+const int32_t *row_order_ids(const int32_t *unq_inv, const int32_t *perm, const int32_t *seg) {
+    return unq_inv ? unq_inv : (perm == nullptr ? seg : nullptr);
+}
+
+// Argument checks, the choice between the row-order table kernels and the voxel-order
+// kernels, and the launches, behind txs_scatter_forward and txs_scatter_forward_resident.
+int scatter_forward_impl(int op, int dtype, const void *feats, const int32_t *unq_inv, const int32_t *perm,
                          const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
-                         const int32_t *heavy_ids, int64_t num_special, void *scratch, void *out,
-                         int32_t *arg, int64_t num_total, int64_t channel, int64_t num_unq,
-                         int64_t max_cnt, void *stream) {
+                         const int32_t *heavy_ids, int64_t num_special, int64_t num_heavy, void *scratch,
+                         int64_t scratch_cells, void *out, int32_t *arg, int64_t num_total, int64_t channel,
+                         int64_t num_unq, int64_t max_cnt, int path, void *stream) {
     if (op != TXS_SUM && op != TXS_MEAN && op != TXS_MAX && op != TXS_MAX_REFTIE)
         return TXS_ERR_UNSUPPORTED;
     if (dtype != TXS_F32 && dtype != TXS_F16 && dtype != TXS_BF16) return TXS_ERR_UNSUPPORTED;
+    if (path != TXS_PATH_AUTO && path != TXS_PATH_VOXEL_ORDER && path != TXS_PATH_TABLE) return TXS_ERR_UNSUPPORTED;
     if (!fits_i32(num_total) || !fits_i32(num_unq) || !fits_i32(channel) || num_special < 0 ||
-        num_special > num_unq)
+        num_special > num_unq || num_heavy < 0 || num_heavy > num_special || scratch_cells < 0)
         return TXS_ERR_INVALID_ARG;
     if (num_unq == 0 || channel == 0) return TXS_OK;
     const bool is_max = op == TXS_MAX || op == TXS_MAX_REFTIE;
     if (!out || !preSum || (is_max && !arg)) return TXS_ERR_INVALID_ARG;
+    const int64_t heavy_cells = num_heavy * channel;  // both below 2^31
+    if (heavy_cells > scratch_cells || (scratch_cells > 0 && !scratch)) return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const int N = (int)num_total, C = (int)channel, U = (int)num_unq;
+
+    // few voxels: reduce in row order into per-workgroup LDS tables (the partial tables
+    // go behind the heavy-voxel table in `scratch`)
+    const int32_t *ids = row_order_ids(unq_inv, perm, seg);
+    if (path != TXS_PATH_VOXEL_ORDER && ids && feats) {
+        const txs_detail::TablePlan tp = txs_detail::table_plan(
+            false, op, dtype, N, C, U, common_alignment({feats, out}));
+        if (tp.use && heavy_cells + tp.partial_cells <= scratch_cells) {
+            unsigned long long *partials = static_cast<unsigned long long *>(scratch) + heavy_cells;
+            return status_of(txs_detail::table_forward(tp, op, dtype, st, feats, ids, preSum, partials, out,
+                                                       arg, N, C, U));
+        }
+    }
+    if (path == TXS_PATH_TABLE) return TXS_ERR_UNSUPPORTED;
+
     // block width the reference would launch for this max_cnt (scatter_kernel.cu:187)
     int ref_log2 = 5;
     while (ref_log2 < 10 && (1LL << ref_log2) < max_cnt) ++ref_log2;
     if (num_total > 0 && (!feats || !seg || !slot_of)) return TXS_ERR_INVALID_ARG;
     if (num_special > 0 && !heavy_ids) return TXS_ERR_INVALID_ARG;
-    hipStream_t st = (hipStream_t)stream;
-    const int N = (int)num_total, C = (int)channel, U = (int)num_unq;
     const int elem = dtype == TXS_F32 ? 4 : 2;
     hipError_t e = hipSuccess;
     if (N > 0) {
@@ -818,7 +854,7 @@ int scatter_forward_impl(int op, int dtype, const void *feats, const int32_t *pe
 
 extern "C" {
 
-int txs_abi_version(void) { return 7; }
+int txs_abi_version(void) { return 8; }
 
 const char *txs_status_string(int status) {
     switch (status) {
@@ -832,25 +868,67 @@ const char *txs_status_string(int status) {
     }
 }
 
+int txs_kernel_name(int backward, int op, int dtype, int64_t num_total, int64_t channel,
+                    int64_t num_unq, int64_t pointer_alignment, int table_allowed, char *buf,
+                    int64_t buf_len) {
+    if (!buf || buf_len < 48) return TXS_ERR_INVALID_ARG;
+    if (op < TXS_SUM || op > TXS_MAX_REFTIE || dtype < TXS_F32 || dtype > TXS_BF16) return TXS_ERR_UNSUPPORTED;
+    if (!fits_i32(num_total) || !fits_i32(channel) || !fits_i32(num_unq) || channel < 1 || num_unq < 1 ||
+        pointer_alignment < 1)
+        return TXS_ERR_INVALID_ARG;
+    static const char *const kOps[] = {"SUM", "MEAN", "MAX", "MAX_REFTIE"};
+    static const char *const kTypes[] = {"F32", "F16", "BF16"};
+    const int elem = dtype == TXS_F32 ? 4 : 2;
+    const void *p = (const void *)(uintptr_t)pointer_alignment;  // stands for the least aligned tensor
+    if (backward && op == TXS_MAX_REFTIE) op = TXS_MAX;
+    if (table_allowed) {
+        const txs_detail::TablePlan tp = txs_detail::table_plan(backward != 0, op, dtype, num_total, channel,
+                                                                num_unq, common_alignment({p}));
+        if (tp.use) {
+            snprintf(buf, (size_t)buf_len, "table_%s_kernel<%s,%d,%s>", backward ? "bwd" : "fwd", kTypes[dtype],
+                     tp.vec_bytes / elem, kOps[op]);
+            return TXS_OK;
+        }
+    }
+    if (backward) {
+        const int chunk = (num_total < (int64_t)kChunkBwdLong * num_unq) ? kChunkBwdShort : kChunkBwdLong;
+        const Geometry geo = make_geometry(num_total, channel, elem, p, p, nullptr, op == TXS_MAX, p, chunk);
+        snprintf(buf, (size_t)buf_len, "scatter_bwd_kernel<%s,%d,%s,%d>", kTypes[dtype], geo.vec_bytes / elem,
+                 kOps[op], chunk);
+    } else {
+        const bool is_max = op == TXS_MAX || op == TXS_MAX_REFTIE;
+        const Geometry geo = make_geometry(num_total, channel, elem, p, p, nullptr, is_max, p, kChunk);
+        snprintf(buf, (size_t)buf_len, "scatter_fwd_kernel<%s,%d,%s>", kTypes[dtype], geo.vec_bytes / elem, kOps[op]);
+    }
+    return TXS_OK;
+}
+
 int txs_default_heavy_threshold(void) { return kHeavyDefault; }
 int txs_chunk_rows(void) { return kChunk; }
 
-int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *perm,
-                        const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
-                        const int32_t *heavy_ids, int64_t num_special, void *scratch, void *out,
-                        int32_t *arg, int64_t num_total, int64_t channel, int64_t num_unq,
-                        int64_t max_cnt, void *stream) {
-    return scatter_forward_impl(op, dtype, feats, perm, seg, preSum, slot_of, heavy_ids, num_special,
-                                scratch, out, arg, num_total, channel, num_unq, max_cnt, stream);
+int64_t txs_scatter_scratch_cells(int64_t num_total, int64_t channel, int64_t num_unq, int64_t num_heavy) {
+    if (!fits_i32(num_total) || !fits_i32(channel) || !fits_i32(num_unq) || num_heavy < 0 || num_heavy > num_unq)
+        return -1;
+    return num_heavy * channel + txs_detail::table_partial_cells(num_total, channel, num_unq);
 }
 
-int txs_scatter_backward(int op, int dtype, const void *grad_out, const int32_t *arg,
-                         const int32_t *perm, const int32_t *seg, const int32_t *preSum,
-                         void *grad_in, int64_t num_total, int64_t channel, int64_t num_unq,
-                         void *stream) {
+int txs_scatter_forward(int op, int dtype, const void *feats, const int32_t *unq_inv, const int32_t *perm,
+                        const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
+                        const int32_t *heavy_ids, int64_t num_special, int64_t num_heavy, void *scratch,
+                        int64_t scratch_cells, void *out, int32_t *arg, int64_t num_total, int64_t channel,
+                        int64_t num_unq, int64_t max_cnt, int path, void *stream) {
+    return scatter_forward_impl(op, dtype, feats, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_special,
+                                num_heavy, scratch, scratch_cells, out, arg, num_total, channel, num_unq,
+                                max_cnt, path, stream);
+}
+
+int txs_scatter_backward(int op, int dtype, const void *grad_out, const int32_t *arg, const int32_t *unq_inv,
+                         const int32_t *perm, const int32_t *seg, const int32_t *preSum, void *grad_in,
+                         int64_t num_total, int64_t channel, int64_t num_unq, int path, void *stream) {
     if (op == TXS_MAX_REFTIE) op = TXS_MAX;  // the backward only reads arg
     if (op != TXS_SUM && op != TXS_MEAN && op != TXS_MAX) return TXS_ERR_UNSUPPORTED;
     if (dtype != TXS_F32 && dtype != TXS_F16 && dtype != TXS_BF16) return TXS_ERR_UNSUPPORTED;
+    if (path != TXS_PATH_AUTO && path != TXS_PATH_VOXEL_ORDER && path != TXS_PATH_TABLE) return TXS_ERR_UNSUPPORTED;
     if (!fits_i32(num_total) || !fits_i32(num_unq) || !fits_i32(channel)) return TXS_ERR_INVALID_ARG;
     if (num_total == 0 || channel == 0) return TXS_OK;
     if (!grad_out || !seg || !grad_in || num_unq <= 0) return TXS_ERR_INVALID_ARG;
@@ -858,6 +936,15 @@ int txs_scatter_backward(int op, int dtype, const void *grad_out, const int32_t 
     if (op == TXS_MEAN && !preSum) return TXS_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const int N = (int)num_total, C = (int)channel, U = (int)num_unq;
+    const int32_t *ids = row_order_ids(unq_inv, perm, seg);
+    if (path != TXS_PATH_VOXEL_ORDER && ids) {
+        // few voxels: upstream rows staged in LDS, input gradient written in row order
+        const txs_detail::TablePlan tp = txs_detail::table_plan(
+            true, op, dtype, N, C, U, common_alignment({grad_out, grad_in, op == TXS_MAX ? (const void *)arg : nullptr}));
+        if (tp.use)
+            return status_of(txs_detail::table_backward(tp, op, dtype, st, grad_out, arg, ids, preSum, grad_in, N, C, U));
+    }
+    if (path == TXS_PATH_TABLE) return TXS_ERR_UNSUPPORTED;
     const int elem = dtype == TXS_F32 ? 4 : 2;
     // short runs on average -> the short chunk; long runs -> the long one
     const int chunk = ((long)N < (long)kChunkBwdLong * U) ? kChunkBwdShort : kChunkBwdLong;
@@ -913,27 +1000,28 @@ int txs_resident_table_init(void) {
     return resident_table(&table);
 }
 
-int txs_scatter_forward_resident(int op, int dtype, const void *feats, const int32_t *perm,
-                                 const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
-                                 const int32_t *heavy_ids, int64_t num_special, int64_t num_heavy,
-                                 void *out, int32_t *arg, int64_t num_total, int64_t channel,
-                                 int64_t num_unq, int64_t max_cnt, void *stream) {
+int txs_scatter_forward_resident(int op, int dtype, const void *feats, const int32_t *unq_inv,
+                                 const int32_t *perm, const int32_t *seg, const int32_t *preSum,
+                                 const int32_t *slot_of, const int32_t *heavy_ids, int64_t num_special,
+                                 int64_t num_heavy, void *out, int32_t *arg, int64_t num_total, int64_t channel,
+                                 int64_t num_unq, int64_t max_cnt, int path, void *stream) {
     if (!fits_i32(channel) || !fits_i32(num_unq) || num_heavy < 0 || num_heavy > num_special ||
         num_special > num_unq)
         return TXS_ERR_INVALID_ARG;
     const int64_t cells = num_heavy * channel;  // both below 2^31: no overflow
     if (cells > kResidentCells) return TXS_ERR_TOO_LARGE;
     unsigned long long *table = nullptr;
+    const int rc = resident_table(&table);
+    if (rc != TXS_OK) return rc;
     if (cells > 0) {
-        const int rc = resident_table(&table);
-        if (rc != TXS_OK) return rc;
         // the table is shared by every call on this GPU and keeps what the last one left:
-        // clear the part this call uses (a kernel, so that the call can be captured)
+        // clear the part the heavy voxels use (a kernel, so that the call can be captured)
         clear_cells_kernel<<<dim3(blocks_for(cells)), dim3(kThreads), 0, (hipStream_t)stream>>>(table, cells);
         if (hipGetLastError() != hipSuccess) return TXS_ERR_LAUNCH;
     }
-    return scatter_forward_impl(op, dtype, feats, perm, seg, preSum, slot_of, heavy_ids, num_special,
-                                table, out, arg, num_total, channel, num_unq, max_cnt, stream);
+    return scatter_forward_impl(op, dtype, feats, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_special,
+                                num_heavy, table, kResidentCells, out, arg, num_total, channel, num_unq,
+                                max_cnt, path, stream);
 }
 
 }  // extern "C"

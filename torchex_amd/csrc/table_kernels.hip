@@ -1,0 +1,384 @@
+// Row-order kernels for inputs with few voxels ("table mode").
+//
+// When the whole [U, C] result fits in the LDS of one compute unit, the rows need not be
+// visited in voxel order at all.  Forward: every workgroup streams a contiguous span of
+// feature rows in the order they lie in memory (fully coalesced, no permutation, which
+// matters most for rows narrower than a cache line), reduces them into a private [U, C]
+// table in LDS with LDS atomics (fp32 add; 64-bit max on ordered(value)<<32 | ~row, so the
+// smallest row wins ties), and stores its table as one partial; a second small kernel
+// combines the partials of all workgroups in a fixed order and writes out / arg.  No
+// global atomics, and nothing has to be zero on entry.  Backward: the upstream rows (and
+// arg rows) are staged in LDS once per workgroup and every input-gradient row is produced
+// in row order, so the large tensor is written sequentially.
+//
+// Replaces, for such inputs, the same reference code as the voxel-order kernels:
+// torchex/src/scatter/scatter_kernel.cu:102-171 and the backward arithmetic of
+// torchex/operator_py/scatter_op.py:47-50,74-78,106-111.
+
+#include "txs_common.h"
+
+namespace {
+
+constexpr int kTableThreads = 1024;          // one workgroup per compute unit
+constexpr int kTableLdsBudget = 144 * 1024;  // bytes of LDS a table may take (160 KB per CU on gfx950)
+constexpr int kTableUnroll = 4;              // rows per lane in flight
+constexpr int kReduceSplit = 16;             // lanes that share the partials of one output cell
+
+template <bool kMax>
+struct CellOf {
+    using type = float;
+};
+template <>
+struct CellOf<true> {
+    using type = unsigned long long;
+};
+
+// ------------------------------------------------------------------ forward --
+
+template <class TR, int VEC, int OP>
+__global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
+    const typename TR::raw *__restrict__ feats, const int *__restrict__ inv,
+    void *__restrict__ partials, int N, int C, int U, int lpr_log2, int stride, int rows_per_wg) {
+    using raw = typename TR::raw;
+    constexpr bool kMax = OP == TXS_MAX;
+    using Cell = typename CellOf<kMax>::type;
+    extern __shared__ unsigned long long table_lds[];
+    Cell *tbl = reinterpret_cast<Cell *>(table_lds);
+    const int cells = U * stride;
+    for (int i = threadIdx.x; i < cells; i += kTableThreads) tbl[i] = Cell(0);
+    __syncthreads();
+
+    const int lane_in = (int)threadIdx.x & ((1 << lpr_log2) - 1);
+    const int g = (int)threadIdx.x >> lpr_log2;
+    const int G = kTableThreads >> lpr_log2;
+    const int col = lane_in * VEC;
+    const long r0 = (long)blockIdx.x * rows_per_wg;
+    const int r_end = (int)min((long)N, r0 + rows_per_wg);
+    if (col < C) {
+        for (int rb = (int)r0 + g; rb < r_end; rb += G * kTableUnroll) {
+            int u[kTableUnroll];
+            Pack<raw, VEC> v[kTableUnroll];
+#pragma unroll
+            for (int k = 0; k < kTableUnroll; ++k) {
+                const int r = min(rb + k * G, r_end - 1);  // slots past the span re-load its last row
+                u[k] = inv[r] & kIdMask;
+                v[k] = ld_stream<raw, VEC>(feats + (size_t)r * C + col);
+            }
+#pragma unroll
+            for (int k = 0; k < kTableUnroll; ++k) {
+                const int r = rb + k * G;
+                if (r >= r_end || (unsigned)u[k] >= (unsigned)U) continue;
+                Cell *dst = tbl + u[k] * stride + col;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float x = TR::to_f(v[k].v[e]);
+                    if constexpr (kMax) {
+                        if (x == x)  // NaN never wins
+                            __hip_atomic_fetch_max(dst + e,
+                                                   ((unsigned long long)ordered_bits(x) << 32) |
+                                                       (unsigned long long)(0xffffffffu - (unsigned)r),
+                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    } else {
+                        __hip_atomic_fetch_add(dst + e, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    // this workgroup's partial: [U, C] cells, dense
+    Cell *part = reinterpret_cast<Cell *>(partials) + (size_t)blockIdx.x * U * C;
+    const int total = U * C;
+    for (int i = threadIdx.x; i < total; i += kTableThreads) {
+        const int uu = i / C, c = i - uu * C;
+        part[i] = tbl[uu * stride + c];
+    }
+}
+
+// out / arg from the partial tables: one output cell per group of kReduceSplit lanes, the
+// partials combined in workgroup order (a fixed order: sums repeat from run to run for a
+// given launch geometry).
+template <class TR, int OP>
+__global__ __launch_bounds__(kThreads) void table_reduce_kernel(
+    const typename TR::raw *__restrict__ feats, const void *__restrict__ partials,
+    const int *__restrict__ preSum, typename TR::raw *__restrict__ out, int *__restrict__ arg,
+    int num_parts, int N, int C, int U) {
+    constexpr bool kMax = OP == TXS_MAX;
+    using Cell = typename CellOf<kMax>::type;
+    constexpr int kCellsPerWg = kThreads / kReduceSplit;
+    __shared__ Cell part_s[kReduceSplit][kCellsPerWg];
+    const int cl = (int)threadIdx.x % kCellsPerWg, wl = (int)threadIdx.x / kCellsPerWg;
+    const long cell = (long)blockIdx.x * kCellsPerWg + cl;
+    const long total = (long)U * C;
+    const Cell *p = reinterpret_cast<const Cell *>(partials);
+    Cell acc = Cell(0);
+    if (cell < total) {
+        for (int w = wl; w < num_parts; w += kReduceSplit) {
+            const Cell x = p[(size_t)w * total + cell];
+            if constexpr (kMax) acc = x > acc ? x : acc; else acc += x;
+        }
+    }
+    part_s[wl][cl] = acc;
+    __syncthreads();
+    if (wl != 0 || cell >= total) return;
+#pragma unroll
+    for (int k = 1; k < kReduceSplit; ++k) {
+        const Cell x = part_s[k][cl];
+        if constexpr (kMax) acc = x > acc ? x : acc; else acc += x;
+    }
+    const int u = (int)(cell / C), c = (int)(cell - (long)u * C);
+    if constexpr (kMax) {
+        const unsigned row = 0xffffffffu - (unsigned)(acc & 0xffffffffull);
+        if (acc == 0ull || row >= (unsigned)N) {  // no rows, or only NaN: the reference's init pair
+            out[cell] = TR::lowest();
+            arg[cell] = -1;
+        } else {
+            out[cell] = feats[(size_t)row * C + c];  // exact bits of the winner (sign of a zero included)
+            arg[cell] = (int)row;
+        }
+    } else {
+        float s = acc;
+        if (OP == TXS_MEAN) s = s / (float)(preSum[u + 1] - preSum[u]);  // 0/0 for an empty voxel, as the reference
+        out[cell] = TR::from_f(s);
+    }
+}
+
+// ----------------------------------------------------------------- backward --
+
+template <class TR, int VEC, int OP>
+__global__ __launch_bounds__(kTableThreads) void table_bwd_kernel(
+    const typename TR::raw *__restrict__ g, const int *__restrict__ arg, const int *__restrict__ inv,
+    const int *__restrict__ preSum, typename TR::raw *__restrict__ gin, int N, int C, int U,
+    int lpr_log2, int stride, int rows_per_wg) {
+    using raw = typename TR::raw;
+    extern __shared__ unsigned long long table_lds[];
+    raw *gt = reinterpret_cast<raw *>(table_lds);
+    // arg rows follow the upstream rows, 32-byte aligned
+    int *at = reinterpret_cast<int *>(reinterpret_cast<char *>(table_lds) +
+                                      (((size_t)U * stride * sizeof(raw) + 31) & ~(size_t)31));
+    const int total = U * C;
+    for (int i = threadIdx.x; i < total; i += kTableThreads) {
+        const int uu = i / C, c = i - uu * C;
+        raw x = g[i];
+        if (OP == TXS_MEAN)  // one division per output cell, as (g / unq_cnts) in the reference
+            x = TR::from_f(TR::to_f(x) / (float)(preSum[uu + 1] - preSum[uu]));
+        gt[uu * stride + c] = x;
+        if (OP == TXS_MAX) at[uu * stride + c] = arg[i];
+    }
+    __syncthreads();
+
+    const int lane_in = (int)threadIdx.x & ((1 << lpr_log2) - 1);
+    const int grp = (int)threadIdx.x >> lpr_log2;
+    const int G = kTableThreads >> lpr_log2;
+    const int col = lane_in * VEC;
+    if (col >= C) return;
+    const long r0 = (long)blockIdx.x * rows_per_wg;
+    const int r_end = (int)min((long)N, r0 + rows_per_wg);
+    for (int rb = (int)r0 + grp; rb < r_end; rb += G * kTableUnroll) {
+        int u[kTableUnroll];
+#pragma unroll
+        for (int k = 0; k < kTableUnroll; ++k) u[k] = inv[min(rb + k * G, r_end - 1)] & kIdMask;
+#pragma unroll
+        for (int k = 0; k < kTableUnroll; ++k) {
+            const int r = rb + k * G;
+            if (r >= r_end) continue;
+            Pack<raw, VEC> o;
+            if ((unsigned)u[k] < (unsigned)U) {
+                o = *reinterpret_cast<const Pack<raw, VEC> *>(gt + u[k] * stride + col);
+                if (OP == TXS_MAX) {
+                    const Pack<int, VEC> a = *reinterpret_cast<const Pack<int, VEC> *>(at + u[k] * stride + col);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) o.v[e] = (a.v[e] == r) ? o.v[e] : TR::zero();
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) o.v[e] = TR::zero();
+            }
+            st_stream<raw, VEC>(gin + (size_t)r * C + col, o);
+        }
+    }
+}
+
+// ------------------------------------------------------------------- launch --
+
+int table_workgroups(long N) {
+    static int cus = 0;  // compute units of the current device
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    // at least 4096 rows per workgroup: a partial table costs as much as its rows otherwise
+    long w = (N + 4095) / 4096;
+    return (int)(w < 1 ? 1 : (w > cus ? cus : w));
+}
+
+template <class K>
+hipError_t allow_lds(K kernel, unsigned bytes) {
+    if (bytes <= 64 * 1024) return hipSuccess;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+template <class TR, int VEC, int OP>
+hipError_t launch_table_fwd(const txs_detail::TablePlan &tp, hipStream_t st, const void *feats,
+                            const int *inv, const int *preSum, void *partials, void *out, int *arg,
+                            int N, int C, int U) {
+    using raw = typename TR::raw;
+    auto kernel = table_fwd_kernel<TR, VEC, OP>;
+    static bool lds_allowed = false;  // per instantiation; the attribute is set for the largest table
+    if (!lds_allowed) {
+        if (allow_lds(kernel, kTableLdsBudget) != hipSuccess) return hipErrorInvalidValue;
+        lds_allowed = true;
+    }
+    kernel<<<dim3(tp.workgroups), dim3(kTableThreads), tp.lds_bytes, st>>>(
+        (const raw *)feats, inv, partials, N, C, U, tp.lpr_log2, tp.stride, tp.rows_per_wg);
+    const long total = (long)U * C;
+    constexpr int kCellsPerWg = kThreads / kReduceSplit;
+    table_reduce_kernel<TR, OP><<<dim3((unsigned)((total + kCellsPerWg - 1) / kCellsPerWg)), dim3(kThreads), 0, st>>>(
+        (const raw *)feats, partials, preSum, (raw *)out, arg, tp.workgroups, N, C, U);
+    return hipGetLastError();
+}
+
+template <class TR, int VEC>
+hipError_t launch_table_fwd_op(int op, const txs_detail::TablePlan &tp, hipStream_t st, const void *feats,
+                               const int *inv, const int *preSum, void *partials, void *out, int *arg,
+                               int N, int C, int U) {
+    switch (op) {
+        case TXS_SUM: return launch_table_fwd<TR, VEC, TXS_SUM>(tp, st, feats, inv, preSum, partials, out, arg, N, C, U);
+        case TXS_MEAN: return launch_table_fwd<TR, VEC, TXS_MEAN>(tp, st, feats, inv, preSum, partials, out, arg, N, C, U);
+        default: return launch_table_fwd<TR, VEC, TXS_MAX>(tp, st, feats, inv, preSum, partials, out, arg, N, C, U);
+    }
+}
+
+template <class TR, int VEC, int OP>
+hipError_t launch_table_bwd(const txs_detail::TablePlan &tp, hipStream_t st, const void *g, const int *arg,
+                            const int *inv, const int *preSum, void *gin, int N, int C, int U) {
+    using raw = typename TR::raw;
+    auto kernel = table_bwd_kernel<TR, VEC, OP>;
+    static bool lds_allowed = false;
+    if (!lds_allowed) {
+        if (allow_lds(kernel, kTableLdsBudget) != hipSuccess) return hipErrorInvalidValue;
+        lds_allowed = true;
+    }
+    kernel<<<dim3(tp.workgroups), dim3(kTableThreads), tp.lds_bytes, st>>>(
+        (const raw *)g, arg, inv, preSum, (raw *)gin, N, C, U, tp.lpr_log2, tp.stride, tp.rows_per_wg);
+    return hipGetLastError();
+}
+
+template <class TR, int VEC>
+hipError_t launch_table_bwd_op(int op, const txs_detail::TablePlan &tp, hipStream_t st, const void *g,
+                               const int *arg, const int *inv, const int *preSum, void *gin, int N, int C,
+                               int U) {
+    switch (op) {
+        case TXS_SUM: return launch_table_bwd<TR, VEC, TXS_SUM>(tp, st, g, arg, inv, preSum, gin, N, C, U);
+        case TXS_MEAN: return launch_table_bwd<TR, VEC, TXS_MEAN>(tp, st, g, arg, inv, preSum, gin, N, C, U);
+        default: return launch_table_bwd<TR, VEC, TXS_MAX>(tp, st, g, arg, inv, preSum, gin, N, C, U);
+    }
+}
+
+// elements per lane: the widest vector (16 bytes at most) that divides a row and fits the
+// alignment of every tensor involved
+int table_vec_bytes(long C, int elem, long align) {
+    int vb = 16;
+    while (vb > elem && ((C * elem) % vb != 0 || align % vb != 0)) vb >>= 1;
+    return vb;
+}
+
+}  // namespace
+
+namespace txs_detail {
+
+TablePlan table_plan(bool backward, int op, int dtype, long N, long C, long U, long align) {
+    TablePlan tp{};
+    if (op == TXS_MAX_REFTIE && !backward) return tp;  // the reference's tie key needs voxel order
+    if (op == TXS_MAX_REFTIE) op = TXS_MAX;
+    if (N <= 0 || C <= 0 || U <= 0) return tp;
+    // few voxels, many rows each: a partial table per workgroup must stay small next to its rows
+    if (N < (long)kTableMinRowsPerVoxel * U || N < 16384) return tp;
+    const int elem = dtype == TXS_F32 ? 4 : 2;
+    const int vb = table_vec_bytes(C, elem, align);
+    const int vec = vb / elem;
+    const long lanes = (C + vec - 1) / vec;
+    if (lanes > 64) return tp;
+    int l2 = 0;
+    while ((1L << l2) < lanes) ++l2;
+    long bytes, stride;
+    if (!backward) {
+        const long cell = op == TXS_MAX ? 8 : 4;
+        stride = C + 1;  // odd number of cells per table row: lanes of different rows spread over the banks
+        bytes = U * stride * cell;
+        if (bytes > kTableLdsBudget) {
+            stride = C;
+            bytes = U * stride * cell;
+        }
+    } else {
+        stride = C + vec;  // keeps every row's vectors aligned
+        bytes = ((U * stride * elem + 31) & ~31L) + (op == TXS_MAX ? U * stride * 4 : 0);
+        if (bytes > kTableLdsBudget) {
+            stride = C;
+            bytes = ((U * stride * elem + 31) & ~31L) + (op == TXS_MAX ? U * stride * 4 : 0);
+        }
+    }
+    if (bytes > kTableLdsBudget) return tp;
+    tp.use = true;
+    tp.vec_bytes = vb;
+    tp.lpr_log2 = l2;
+    tp.stride = (int)stride;
+    tp.lds_bytes = (unsigned)((bytes + 15) & ~15L);
+    tp.workgroups = table_workgroups(N);
+    tp.rows_per_wg = (int)((N + tp.workgroups - 1) / tp.workgroups);
+    tp.partial_cells = backward ? 0 : (long)tp.workgroups * U * C;
+    return tp;
+}
+
+long table_partial_cells(long N, long C, long U) {
+    // capacity for whichever operator and dtype asks for the most (8-byte cells either way)
+    long most = 0;
+    for (int op = TXS_SUM; op <= TXS_MAX; ++op)
+        for (int dt = TXS_F32; dt <= TXS_BF16; ++dt) {
+            const TablePlan tp = table_plan(false, op, dt, N, C, U, 16);
+            if (tp.use && tp.partial_cells > most) most = tp.partial_cells;
+        }
+    return most;
+}
+
+hipError_t table_forward(const TablePlan &tp, int op, int dtype, hipStream_t st, const void *feats,
+                         const int *inv, const int *preSum, void *partials, void *out, int *arg, int N,
+                         int C, int U) {
+#define TXS_TAB(TR, VB)                                                                                  \
+    if (tp.vec_bytes == VB)                                                                              \
+        return launch_table_fwd_op<TR, (VB) / (int)sizeof(typename TR::raw)>(op, tp, st, feats, inv, preSum, \
+                                                                             partials, out, arg, N, C, U);
+    if (dtype == TXS_F32) {
+        TXS_TAB(F32, 16) TXS_TAB(F32, 8) TXS_TAB(F32, 4)
+    } else if (dtype == TXS_F16) {
+        TXS_TAB(F16, 16) TXS_TAB(F16, 8) TXS_TAB(F16, 4) TXS_TAB(F16, 2)
+    } else {
+        TXS_TAB(BF16, 16) TXS_TAB(BF16, 8) TXS_TAB(BF16, 4) TXS_TAB(BF16, 2)
+    }
+#undef TXS_TAB
+    return hipErrorInvalidValue;
+}
+
+hipError_t table_backward(const TablePlan &tp, int op, int dtype, hipStream_t st, const void *g,
+                          const int *arg, const int *inv, const int *preSum, void *gin, int N, int C, int U) {
+#define TXS_TAB(TR, VB)                                                                                  \
+    if (tp.vec_bytes == VB)                                                                              \
+        return launch_table_bwd_op<TR, (VB) / (int)sizeof(typename TR::raw)>(op, tp, st, g, arg, inv, preSum, \
+                                                                             gin, N, C, U);
+    if (dtype == TXS_F32) {
+        TXS_TAB(F32, 16) TXS_TAB(F32, 8) TXS_TAB(F32, 4)
+    } else if (dtype == TXS_F16) {
+        TXS_TAB(F16, 16) TXS_TAB(F16, 8) TXS_TAB(F16, 4) TXS_TAB(F16, 2)
+    } else {
+        TXS_TAB(BF16, 16) TXS_TAB(BF16, 8) TXS_TAB(BF16, 4) TXS_TAB(BF16, 2)
+    }
+#undef TXS_TAB
+    return hipErrorInvalidValue;
+}
+
+}  // namespace txs_detail

@@ -28,6 +28,15 @@ namespace {
 #ifndef TXS_BATCH_BWD
 #define TXS_BATCH_BWD TXS_BATCH
 #endif
+#ifndef TXS_BATCH_HALF
+#define TXS_BATCH_HALF TXS_BATCH
+#endif
+#ifndef TXS_BATCH_BWD_HALF
+#define TXS_BATCH_BWD_HALF TXS_BATCH_BWD
+#endif
+#ifndef TXS_HALF_VEC_BYTES
+#define TXS_HALF_VEC_BYTES 8
+#endif
 #ifndef TXS_NT_LOADS
 #define TXS_NT_LOADS 1
 #endif
@@ -41,8 +50,11 @@ constexpr int kChunkBwdShort = TXS_CHUNK_BWD_SHORT;  // backward kernel, mean ru
 constexpr int kChunkBwdLong = TXS_CHUNK;             // backward kernel, longer runs
 constexpr int kBatchBwd = TXS_BATCH_BWD;
 constexpr int kBatch = TXS_BATCH;    // rows per load batch of a lane group (two batches in flight)
-constexpr int kHalfVecBytes = 8;     // bytes one lane moves per row for fp16 / bf16
+constexpr int kBatchHalf = TXS_BATCH_HALF;         // the same for the 2-byte types
+constexpr int kBatchBwdHalf = TXS_BATCH_BWD_HALF;
+constexpr int kHalfVecBytes = TXS_HALF_VEC_BYTES;  // bytes one lane moves per row for fp16 / bf16
 constexpr int kHeavyDefault = 64;    // voxels above this many rows use the atomic path
+constexpr int kTableMinRowsPerVoxel = 512;  // table mode needs at least this many rows per voxel on average
 constexpr int kSpecialBit = (int)0x80000000;
 constexpr int kIdMask = 0x7fffffff;
 
@@ -201,5 +213,27 @@ long scan_tiles(long n_out);
 // out[i] = sum_{k<i} in[k] for i in [0, n_out), where in[k] = 0 for k >= n_in; in
 // and out may alias.  Three launches on `st`, no inter-block waiting.
 hipError_t exclusive_scan(const int *in, long n_in, int *out, long n_out, int *ws, hipStream_t st);
+
+
+// Row-order "table mode" for inputs with few voxels (table_kernels.hip): whether it
+// applies to a call and with which launch geometry.
+struct TablePlan {
+    bool use;            // false: the call takes the voxel-order kernels
+    int vec_bytes;       // bytes one lane moves per row
+    int lpr_log2;        // log2(lanes per row)
+    int stride;          // cells (forward) or elements (backward) per table row in LDS
+    unsigned lds_bytes;  // dynamic LDS per workgroup
+    int workgroups, rows_per_wg;
+    long partial_cells;  // 8-byte cells of workspace the forward needs for its partial tables
+};
+// `align`: alignment in bytes shared by every tensor of the call (a power of two).
+TablePlan table_plan(bool backward, int op, int dtype, long N, long C, long U, long align);
+// Workspace (8-byte cells) that lets any operator / dtype of these extents run in table mode; 0 if none can.
+long table_partial_cells(long N, long C, long U);
+hipError_t table_forward(const TablePlan &tp, int op, int dtype, hipStream_t st, const void *feats,
+                         const int *inv, const int *preSum, void *partials, void *out, int *arg, int N,
+                         int C, int U);
+hipError_t table_backward(const TablePlan &tp, int op, int dtype, hipStream_t st, const void *g,
+                          const int *arg, const int *inv, const int *preSum, void *gin, int N, int C, int U);
 
 }  // namespace txs_detail

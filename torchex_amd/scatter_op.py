@@ -60,6 +60,10 @@ class ScatterData:
     smallest row index; ``None`` (default) picks ``"reference"`` for grouped input and
     ``"first"`` otherwise.  The rule in force is kept as ``self.max_tie_rule``.
 
+    ``path`` (attribute, default ``scatter_ext.PATH_AUTO``) lets a caller force the
+    voxel-order kernels (``PATH_VOXEL_ORDER``) or the row-order table kernels for inputs
+    with few voxels (``PATH_TABLE``; raises where they do not apply).
+
     ``assume_sorted=True`` states that ``unq_inv`` is already grouped (the order the
     reference requires): the sort is then not queued at all; the statement is
     verified on the device and an unsorted ``unq_inv`` raises.
@@ -90,6 +94,10 @@ class ScatterData:
         assert stats[5] == 0, "unq_cnts is not the histogram of unq_inv"
         self.num_total = flat.shape[0]
         self.is_sorted = self.perm is None
+        # voxel id of every row in row order, for the row-order (few-voxel) kernels; grouped
+        # rows need none: their per-position ids are the row-order ids
+        self.row_ids = None if self.is_sorted else flat
+        self.path = scatter_ext.PATH_AUTO
         self.max_tie_rule = _resolve_tie_rule(max_tie_rule, self.is_sorted)
         self.max_cnt = int(stats[2])
         self.num_special = int(stats[3])
@@ -118,6 +126,8 @@ class ScatterData:
         self.unq_cnts = cnts.unsqueeze(-1)
         self.num_total = flat.shape[0]
         self.is_sorted = self.perm is None
+        self.row_ids = None if self.is_sorted else self.unq_inv
+        self.path = scatter_ext.PATH_AUTO
         self.max_tie_rule = _resolve_tie_rule(max_tie_rule, self.is_sorted)
         self.max_cnt = int(stats[2])
         self.num_special = int(stats[3])
@@ -140,16 +150,26 @@ class ScatterData:
         return self
 
     def scratch(self, channel):
-        """Zeroed table the heavy voxels are merged in (one row each); the kernels leave it
-        zeroed again, so a buffer is kept for reuse -- one per channel count and per
-        stream: calls queued on one stream are ordered, and forwards that run
-        concurrently on different streams each get a table of their own."""
+        """Forward workspace: the zeroed table the heavy voxels are merged in (one row each,
+        left zeroed again by the kernels) and, for inputs with few voxels, room for the
+        partial tables of the row-order kernels.  A buffer is kept for reuse -- one per
+        channel count and per stream: calls queued on one stream are ordered, and forwards
+        that run concurrently on different streams each get a workspace of their own."""
         key = (channel, torch.cuda.current_stream(self.seg.device).stream_id)
         buf = self._scratch.get(key)
         if buf is None:
-            buf = scatter_ext.make_scratch(self.num_heavy, channel, self.seg)
+            buf = scatter_ext.make_scratch(self.num_total, channel, self.num_unq, self.num_heavy, self.seg)
             self._scratch[key] = buf
         return buf
+
+    def forward_args(self, channel):
+        """Plan arguments of ``scatter_ext.forward`` after ``(op, feats)``."""
+        return (self.row_ids, self.perm, self.seg, self.preSum, self.slot_of, self.heavy_ids, self.num_heavy,
+                self.scratch(channel), self.max_cnt, self.path)
+
+    def backward_args(self):
+        """Plan arguments of ``scatter_ext.backward`` after ``(op, grad_out, arg)``."""
+        return (self.row_ids, self.perm, self.seg, self.preSum, self.num_total, self.path)
 
 
 def _check_feats(feats, data):
@@ -162,13 +182,11 @@ def _check_feats(feats, data):
 
 def _forward(op, feats, data):
     _check_feats(feats, data)
-    return scatter_ext.forward(op, feats, data.perm, data.seg, data.preSum, data.slot_of,
-                               data.heavy_ids, data.scratch(feats.shape[1]), data.max_cnt)
+    return scatter_ext.forward(op, feats, *data.forward_args(feats.shape[1]))
 
 
 def _backward(op, g, arg, data):
-    return scatter_ext.backward(op, g.contiguous(), arg, data.perm, data.seg, data.preSum,
-                                data.num_total)
+    return scatter_ext.backward(op, g.contiguous(), arg, *data.backward_args())
 
 
 class ScatterSumFunction(Function):
