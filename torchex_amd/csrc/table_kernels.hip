@@ -4,7 +4,7 @@
 // visited in voxel order at all.  Forward: every workgroup streams a contiguous span of
 // feature rows in the order they lie in memory (fully coalesced, no permutation, which
 // matters most for rows narrower than a cache line), reduces them into a private [U, C]
-// table in LDS with LDS atomics (fp32 add; 64-bit max on ordered(value)<<32 | ~row, so the
+// table in LDS with LDS atomics (fp64 add; 64-bit max on ordered(value)<<32 | ~row, so the
 // smallest row wins ties), and stores its table as one partial; a second small kernel
 // combines the partials of all workgroups in a fixed order and writes out / arg.  No
 // global atomics, and nothing has to be zero on entry.  Backward: the upstream rows (and
@@ -21,19 +21,26 @@ namespace {
 
 constexpr int kTableThreads = 1024;          // one workgroup per compute unit
 constexpr int kTableLdsBudget = 144 * 1024;  // bytes of LDS a table may take (160 KB per CU on gfx950)
-constexpr int kTableUnroll = 4;              // rows per lane in flight
-constexpr int kReduceSplit = 16;             // lanes that share the partials of one output cell
-
-template <bool kMax>
-struct CellOf {
-    using type = float;
-};
-template <>
-struct CellOf<true> {
-    using type = unsigned long long;
-};
+#ifndef TXS_TABLE_MAX_WGS
+#define TXS_TABLE_MAX_WGS 1024
+#endif
+#ifndef TXS_TABLE_UNROLL
+#define TXS_TABLE_UNROLL 4
+#endif
+constexpr int kTableUnroll = TXS_TABLE_UNROLL;  // rows per lane in flight
+constexpr int kReduceThreads = 1024;
+constexpr int kReduceSplit = 64;             // lanes that share the partials of one output cell
+constexpr int kReduceLoads = 4;              // partials each of them has in flight
 
 // ------------------------------------------------------------------ forward --
+//
+// LDS cells are 8 bytes for every operator: a packed (ordered value, ~row) word for max,
+// a double for sum / mean.  The fp64 cell is a matter of speed, not of accuracy: on this
+// part an LDS fp32 atomic add retires about one lane every three cycles, whatever the
+// addresses, while fp64 and integer LDS atomics run seven times faster (2M rows of 16
+// channels into 1024 voxels: 164 us with fp32 cells, 26 us with fp64 cells, 20 us for the
+// load stream alone).  A workgroup's partial is stored as fp32 (sum / mean) or as the
+// packed word (max).
 
 template <class TR, int VEC, int OP>
 __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
@@ -41,11 +48,11 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
     void *__restrict__ partials, int N, int C, int U, int lpr_log2, int stride, int rows_per_wg) {
     using raw = typename TR::raw;
     constexpr bool kMax = OP == TXS_MAX;
-    using Cell = typename CellOf<kMax>::type;
     extern __shared__ unsigned long long table_lds[];
-    Cell *tbl = reinterpret_cast<Cell *>(table_lds);
+    unsigned long long *tkey = table_lds;
+    double *tsum = reinterpret_cast<double *>(table_lds);
     const int cells = U * stride;
-    for (int i = threadIdx.x; i < cells; i += kTableThreads) tbl[i] = Cell(0);
+    for (int i = threadIdx.x; i < cells; i += kTableThreads) tkey[i] = 0ull;  // +0.0 as a double
     __syncthreads();
 
     const int lane_in = (int)threadIdx.x & ((1 << lpr_log2) - 1);
@@ -68,62 +75,93 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
             for (int k = 0; k < kTableUnroll; ++k) {
                 const int r = rb + k * G;
                 if (r >= r_end || (unsigned)u[k] >= (unsigned)U) continue;
-                Cell *dst = tbl + u[k] * stride + col;
+                const int cell = u[k] * stride + col;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     const float x = TR::to_f(v[k].v[e]);
                     if constexpr (kMax) {
                         if (x == x)  // NaN never wins
-                            __hip_atomic_fetch_max(dst + e,
+                            __hip_atomic_fetch_max(tkey + cell + e,
                                                    ((unsigned long long)ordered_bits(x) << 32) |
                                                        (unsigned long long)(0xffffffffu - (unsigned)r),
                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                     } else {
-                        __hip_atomic_fetch_add(dst + e, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        __hip_atomic_fetch_add(tsum + cell + e, (double)x, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_WORKGROUP);
                     }
                 }
             }
         }
     }
     __syncthreads();
-    // this workgroup's partial: [U, C] cells, dense
-    Cell *part = reinterpret_cast<Cell *>(partials) + (size_t)blockIdx.x * U * C;
+    // this workgroup's partial: [U, C], dense
     const int total = U * C;
-    for (int i = threadIdx.x; i < total; i += kTableThreads) {
-        const int uu = i / C, c = i - uu * C;
-        part[i] = tbl[uu * stride + c];
+    if constexpr (kMax) {
+        unsigned long long *part = reinterpret_cast<unsigned long long *>(partials) + (size_t)blockIdx.x * total;
+        for (int i = threadIdx.x; i < total; i += kTableThreads) {
+            const int uu = i / C;
+            part[i] = tkey[uu * stride + (i - uu * C)];
+        }
+    } else {
+        float *part = reinterpret_cast<float *>(partials) + (size_t)blockIdx.x * total;
+        for (int i = threadIdx.x; i < total; i += kTableThreads) {
+            const int uu = i / C;
+            part[i] = (float)tsum[uu * stride + (i - uu * C)];
+        }
     }
 }
 
 // out / arg from the partial tables: one output cell per group of kReduceSplit lanes, the
-// partials combined in workgroup order (a fixed order: sums repeat from run to run for a
-// given launch geometry).
+// partials combined in workgroup order (a fixed order: for a given launch geometry only
+// the order of the atomic adds inside a workgroup varies from run to run).
 template <class TR, int OP>
-__global__ __launch_bounds__(kThreads) void table_reduce_kernel(
+__global__ __launch_bounds__(kReduceThreads) void table_reduce_kernel(
     const typename TR::raw *__restrict__ feats, const void *__restrict__ partials,
     const int *__restrict__ preSum, typename TR::raw *__restrict__ out, int *__restrict__ arg,
     int num_parts, int N, int C, int U) {
     constexpr bool kMax = OP == TXS_MAX;
-    using Cell = typename CellOf<kMax>::type;
-    constexpr int kCellsPerWg = kThreads / kReduceSplit;
-    __shared__ Cell part_s[kReduceSplit][kCellsPerWg];
+    using Cell = typename std::conditional<kMax, unsigned long long, float>::type;  // as the forward stored it
+    using Acc = typename std::conditional<kMax, unsigned long long, double>::type;
+    constexpr int kCellsPerWg = kReduceThreads / kReduceSplit;
+    __shared__ Acc part_s[kReduceSplit][kCellsPerWg];
     const int cl = (int)threadIdx.x % kCellsPerWg, wl = (int)threadIdx.x / kCellsPerWg;
     const long cell = (long)blockIdx.x * kCellsPerWg + cl;
     const long total = (long)U * C;
     const Cell *p = reinterpret_cast<const Cell *>(partials);
-    Cell acc = Cell(0);
+    Acc acc = Acc(0);
     if (cell < total) {
-        for (int w = wl; w < num_parts; w += kReduceSplit) {
-            const Cell x = p[(size_t)w * total + cell];
-            if constexpr (kMax) acc = x > acc ? x : acc; else acc += x;
+        // kReduceLoads independent loads in flight per lane
+        for (int w0 = wl; w0 < num_parts; w0 += kReduceSplit * kReduceLoads) {
+            Cell x[kReduceLoads];
+#pragma unroll
+            for (int k = 0; k < kReduceLoads; ++k) {
+                const int w = w0 + k * kReduceSplit;
+                x[k] = w < num_parts ? p[(size_t)w * total + cell] : Cell(0);
+            }
+#pragma unroll
+            for (int k = 0; k < kReduceLoads; ++k) {
+                if constexpr (kMax) acc = (Acc)x[k] > acc ? (Acc)x[k] : acc; else acc += (Acc)x[k];
+            }
         }
     }
     part_s[wl][cl] = acc;
     __syncthreads();
+    // second level in a fixed order: lanes 0..7 of a cell each fold 8 of the 64 values, lane 0 folds those
+    if (wl < 8) {
+        acc = part_s[wl * 8][cl];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) {
+            const Acc x = part_s[wl * 8 + k][cl];
+            if constexpr (kMax) acc = x > acc ? x : acc; else acc += x;
+        }
+    }
+    __syncthreads();
+    if (wl < 8) part_s[wl][cl] = acc;
+    __syncthreads();
     if (wl != 0 || cell >= total) return;
 #pragma unroll
-    for (int k = 1; k < kReduceSplit; ++k) {
-        const Cell x = part_s[k][cl];
+    for (int k = 1; k < 8; ++k) {
+        const Acc x = part_s[k][cl];
         if constexpr (kMax) acc = x > acc ? x : acc; else acc += x;
     }
     const int u = (int)(cell / C), c = (int)(cell - (long)u * C);
@@ -137,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void table_reduce_kernel(
             arg[cell] = (int)row;
         }
     } else {
-        float s = acc;
+        float s = (float)acc;
         if (OP == TXS_MEAN) s = s / (float)(preSum[u + 1] - preSum[u]);  // 0/0 for an empty voxel, as the reference
         out[cell] = TR::from_f(s);
     }
@@ -213,7 +251,8 @@ int table_workgroups(long N) {
     }
     // at least 4096 rows per workgroup: a partial table costs as much as its rows otherwise
     long w = (N + 4095) / 4096;
-    return (int)(w < 1 ? 1 : (w > cus ? cus : w));
+    const long most = cus < TXS_TABLE_MAX_WGS ? cus : TXS_TABLE_MAX_WGS;
+    return (int)(w < 1 ? 1 : (w > most ? most : w));
 }
 
 template <class K>
@@ -237,8 +276,8 @@ hipError_t launch_table_fwd(const txs_detail::TablePlan &tp, hipStream_t st, con
     kernel<<<dim3(tp.workgroups), dim3(kTableThreads), tp.lds_bytes, st>>>(
         (const raw *)feats, inv, partials, N, C, U, tp.lpr_log2, tp.stride, tp.rows_per_wg);
     const long total = (long)U * C;
-    constexpr int kCellsPerWg = kThreads / kReduceSplit;
-    table_reduce_kernel<TR, OP><<<dim3((unsigned)((total + kCellsPerWg - 1) / kCellsPerWg)), dim3(kThreads), 0, st>>>(
+    constexpr int kCellsPerWg = kReduceThreads / kReduceSplit;
+    table_reduce_kernel<TR, OP><<<dim3((unsigned)((total + kCellsPerWg - 1) / kCellsPerWg)), dim3(kReduceThreads), 0, st>>>(
         (const raw *)feats, partials, preSum, (raw *)out, arg, tp.workgroups, N, C, U);
     return hipGetLastError();
 }
@@ -308,7 +347,7 @@ TablePlan table_plan(bool backward, int op, int dtype, long N, long C, long U, l
     while ((1L << l2) < lanes) ++l2;
     long bytes, stride;
     if (!backward) {
-        const long cell = op == TXS_MAX ? 8 : 4;
+        const long cell = 8;  // every operator keeps 8-byte cells in LDS
         stride = C + 1;  // odd number of cells per table row: lanes of different rows spread over the banks
         bytes = U * stride * cell;
         if (bytes > kTableLdsBudget) {
