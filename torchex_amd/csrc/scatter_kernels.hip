@@ -99,7 +99,9 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     // Partials of heavy voxels: two slots per lane group (a chunk can touch at
     // most two heavy runs, one at each end), combined across the workgroup
     // before anything goes to the global scratch table.
-    using SlotT = typename std::conditional<kMax, unsigned long long, float>::type;
+    // (sum / mean partials are parked as doubles: LDS fp64 atomic adds run several times
+    // faster than fp32 ones on this part)
+    using SlotT = typename std::conditional<kMax, unsigned long long, double>::type;
     int *slot_id = perm_s + (n_seg_s - 1);
     SlotT *slot_val = reinterpret_cast<SlotT *>(lds + ((2 * n_seg_s - 1 + 2 * G + 1) & ~1));
     const int W = VEC << lpr_log2;        // elements per slot
@@ -237,7 +239,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                                            (unsigned long long)(0xffffffffu - (unsigned)idx[k]))
                                         : 0ull;
                 } else {
-                    sv[k] = acc[k];
+                    sv[k] = (double)acc[k];
                 }
             }
         }
@@ -415,7 +417,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
         if constexpr (kMax) {
             if (tot != 0ull) atomicMax(scratch + o, tot);
         } else {
-            unsafeAtomicAdd(reinterpret_cast<float *>(scratch) + o, tot);
+            unsafeAtomicAdd(reinterpret_cast<float *>(scratch) + o, (float)tot);
         }
     }
 }
@@ -456,7 +458,10 @@ __global__ void scatter_finalize_kernel(const typename TR::raw *__restrict__ fea
             out[o] = TR::lowest();
             arg[o] = -1;
         } else {
-            out[o] = feats[(size_t)row * C + c];  // exact bits of the winner
+            // the key carries the winning value itself (exactly: it came from the dtype);
+            // only the sign of a zero was folded away and is read back from the winner
+            const float x = from_ordered_bits((unsigned)(key >> 32));
+            out[o] = x == 0.0f ? feats[(size_t)row * C + c] : TR::from_f(x);
             arg[o] = (int)row;
         }
     } else {
@@ -642,14 +647,14 @@ hipError_t launch_fwd_op(int op, const Geometry &geo, hipStream_t st, const void
     auto o = (raw *)out;
     auto s = (unsigned long long *)scratch;
     dim3 blk(kThreads);
-    const unsigned lds4 = geo.lds_fwd_idx + 4 * geo.lds_slots, lds8 = geo.lds_fwd_idx + 8 * geo.lds_slots;
+    const unsigned lds8 = geo.lds_fwd_idx + 8 * geo.lds_slots;  // 8-byte slot cells for every operator
     switch (op) {
         case TXS_SUM:
-            scatter_fwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, lds4, st>>>(
+            scatter_fwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, lds8, st>>>(
                 f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
             break;
         case TXS_MEAN:
-            scatter_fwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, lds4, st>>>(
+            scatter_fwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, lds8, st>>>(
                 f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
             break;
         case TXS_MAX_REFTIE:

@@ -171,7 +171,9 @@ __global__ __launch_bounds__(kReduceThreads) void table_reduce_kernel(
             out[cell] = TR::lowest();
             arg[cell] = -1;
         } else {
-            out[cell] = feats[(size_t)row * C + c];  // exact bits of the winner (sign of a zero included)
+            // the key carries the winning value; only the sign of a zero is read back from the winner
+            const float x = from_ordered_bits((unsigned)(acc >> 32));
+            out[cell] = x == 0.0f ? feats[(size_t)row * C + c] : TR::from_f(x);
             arg[cell] = (int)row;
         }
     } else {

@@ -160,6 +160,11 @@ __device__ __forceinline__ unsigned ordered_bits(float v) {
     return b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u);
 }
 
+// inverse of ordered_bits (a zero comes back as +0.0)
+__device__ __forceinline__ float from_ordered_bits(unsigned r) {
+    return __uint_as_float((r & 0x80000000u) ? (r ^ 0x80000000u) : ~r);
+}
+
 // ----------------------------------------------------------- workgroup scan --
 
 __device__ __forceinline__ int wave_inclusive_scan(int x) {
