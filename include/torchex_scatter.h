@@ -82,7 +82,8 @@ enum {
     TXS_STAT_COUNT_MISMATCH = 5, /* 1 if the caller's unq_cnts is not the histogram of unq_inv */
     TXS_STAT_NUM_UNQ = 6,      /* number of distinct keys found by txs_unique_runs */
     TXS_STAT_NUM_HEAVY = 7,    /* number of voxels above the heavy threshold (NUM_SPECIAL - NUM_EMPTY) */
-    TXS_STATS_LEN = 8
+    TXS_STAT_NEED_GENERAL = 8, /* txs_plan_build only: 1 if it left the outputs unwritten (see there) */
+    TXS_STATS_LEN = 16
 };
 
 /* Library ABI version (8); bumped when a signature or the meaning of an argument changes. */
@@ -157,6 +158,32 @@ int txs_plan_presum(const int32_t *sorted_keys, int64_t num_total, int64_t num_u
 int txs_plan_special(const int32_t *preSum, int64_t num_unq, int32_t heavy_threshold,
                      const int64_t *unq_cnts, int32_t *slot_of, int32_t *heavy_ids, int32_t *stats,
                      const int32_t *num_unq_dev, int64_t *cnts_out, void *stream);
+
+/* Everything ScatterData.__init__ needs, in one call: order/range flags, the stable
+ * permutation, CSR offsets, special-voxel table, statistics and the flagged per-position
+ * ids (what txs_plan_check, txs_plan_sort, txs_plan_presum, txs_plan_special and
+ * txs_plan_seg_flag produce one after the other).  Up to 2^22 voxels this runs as a
+ * bucket sort -- tile histograms of the high digit of the ids; scan; stable scatter by
+ * bucket; then workgroups that sort a bucket's low digit in LDS and write the bucket's
+ * slice of all outputs -- beyond that it runs the calls named above.
+ * stats [TXS_STATS_LEN] needs no initialisation for up to 2^22 voxels and must be
+ * zero-filled by the caller beyond (zero-filling always is fine); perm is left unwritten when
+ * stats[UNSORTED] stays 0.  unq_cnts may be NULL.  plan_ws: int32 workspace of
+ * txs_plan_workspace_len(num_total, num_unq) entries, 8-byte aligned.
+ * One bucket holding more than 262,144 rows (a few voxels that own most of the rows)
+ * makes the bucket kernels step aside: stats[NEED_GENERAL] is then 1, only
+ * stats[UNSORTED] and stats[OUT_OF_RANGE] are valid, and the caller zero-fills stats
+ * again and calls txs_plan_build_general with the same arguments. */
+int txs_plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
+                   int32_t heavy_threshold, const int64_t *unq_cnts, int32_t *plan_ws,
+                   int32_t *perm, int32_t *seg, int32_t *preSum, int32_t *slot_of,
+                   int32_t *heavy_ids, int32_t *stats, void *stream);
+int64_t txs_plan_workspace_len(int64_t num_total, int64_t num_unq);
+/* The same outputs through the general sequence (any number of voxels, any occupancy). */
+int txs_plan_build_general(const int32_t *unq_inv, int64_t num_total, int64_t num_unq,
+                           int32_t heavy_threshold, const int64_t *unq_cnts, int32_t *plan_ws,
+                           int32_t *perm, int32_t *seg, int32_t *preSum, int32_t *slot_of,
+                           int32_t *heavy_ids, int32_t *stats, void *stream);
 
 /* In place: sorted keys -> seg (sets bit 31 on positions of special voxels). */
 int txs_plan_seg_flag(int32_t *keys_to_seg, int64_t num_total, int64_t num_unq,

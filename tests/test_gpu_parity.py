@@ -1104,3 +1104,20 @@ def test_table_kernels_special_values_and_grouped_rows():
     dl.path = scatter_ext.PATH_TABLE
     with pytest.raises(RuntimeError, match="unsupported"):
         T.scatter_sum(w.feats.to(DEV), dl)
+
+
+def test_plan_with_crowded_buckets_and_the_general_fallback():
+    """Index preparation splits the ids into buckets of consecutive voxels.  A bucket with far
+    more rows than the others is shared by several workgroups; one that holds more than 262,144
+    rows sends the whole plan to the general radix passes.  Both give the same plan as the oracle."""
+    g = torch.Generator().manual_seed(13)
+    U, C = 5000, 8                      # 13 bits of id: buckets of 32 consecutive voxels
+    for name, crowd in (("shared bucket", 100_000), ("giant bucket", 300_000)):
+        N = crowd + 120_000
+        inv = torch.randint(0, U, (N,), generator=g)
+        hot = torch.randperm(N, generator=g)[:crowd]
+        inv[hot] = torch.randint(3, 9, (crowd,), generator=g)      # voxels 3..8 take `crowd` rows
+        inv[:U] = torch.arange(U)
+        feats = torch.randint(-4, 5, (N, C), generator=g).float()
+        data = run_case(name, feats, inv, torch.bincount(inv, minlength=U))
+        assert data.max_cnt > crowd // 7 and data.perm is not None

@@ -335,6 +335,411 @@ __global__ void seg_from_presum_kernel(const int *__restrict__ preSum, long n, i
     seg[j] = lo | flag;
 }
 
+// ------------------------------------------------ two-level plan (bucket sort) --
+//
+// For up to 2^22 voxels the whole index preparation is three kernels and a scan:
+//   (1) bucket_hist_kernel: per tile of 8192 rows, the histogram of the HIGH digit of the
+//       voxel id (the "bucket") and the tile's order / range flags;
+//   (2) exclusive scan of the digit-major histogram;
+//   (3) bucket_scatter_kernel: flags of the whole input, bucket boundaries, and the stable
+//       scatter of (id, row) pairs by bucket (wave-ballot ranking);
+//   (4) bucket_plan_kernel: counting sort of every bucket by the LOW digit (<= 11 bits) in
+//       LDS, which at the same time yields the bucket's slice of everything else the plan
+//       holds: CSR offsets, per-voxel counts (checked against the caller's), the
+//       special-voxel table and its slots, max_cnt, and the flagged per-position ids
+//       written next to the permutation.  A bucket of more than 8192 rows is shared by up
+//       to 16 workgroups: each counts the whole bucket (LDS integer atomics) and the rows
+//       in front of its own slice, then places its slice.
+// Ids of at most 11 bits need no low digit: (3) already gives the final order, and the
+// elementwise kernels used by the general sequence finish the plan.
+// Measured alternatives (1M ids of 19 bits, 0.13 ms per plan as built): an 11-bit bucket digit
+// makes the scatter write 16-byte runs and costs 30 us instead of 20; folding the scan into
+// the scatter (every workgroup adding up the tile histograms itself) saves two launches but
+// costs more than it saves from about 100 tiles on; per-voxel instead of per-row offset
+// bookkeeping in (4) makes no difference.
+
+constexpr int kBucketHighBits = 8;
+constexpr int kBucketLowBitsMax = 11;   // also the largest high digit
+constexpr int kBucketBitsMax = 22;
+constexpr int kHistThreads = 512, kHistItems = 16;
+constexpr int kHistTile = kHistThreads * kHistItems;  // 8192 rows per tile
+constexpr int kHistWaves = kHistThreads / 64;
+constexpr int kBktItems = 16;
+constexpr int kBktChunk = kThreads * kBktItems;        // 4096 rows per placement round
+constexpr int kBktWaves = kThreads / 64;
+constexpr int kBktSlice = 2 * kBktChunk;               // rows one workgroup places
+constexpr int kBktMaxSlices = 16;                      // workgroups per bucket at most
+constexpr int kFlagUnsorted = 1, kFlagOutOfRange = 2;
+
+// hist: [high_bins][n_tiles] digit-major (the order its exclusive scan needs); tile_flags: [n_tiles]
+__global__ __launch_bounds__(kHistThreads) void bucket_hist_kernel(
+    const int *__restrict__ inv, long n, int U, int low_bits, int high_bins, int *__restrict__ hist,
+    int *__restrict__ tile_flags, int n_tiles) {
+    __shared__ int h[1 << kBucketLowBitsMax];
+    __shared__ int s_flags;
+    for (int d = threadIdx.x; d < high_bins; d += kHistThreads) h[d] = 0;
+    if (threadIdx.x == 0) s_flags = 0;
+    __syncthreads();
+    const long base = (long)blockIdx.x * kHistTile;
+    int v[kHistItems];
+#pragma unroll
+    for (int it = 0; it < kHistItems; ++it) {
+        const long i = base + (long)it * kHistThreads + threadIdx.x;
+        v[it] = i < n ? inv[i] : 0x7fffffff;
+    }
+    bool bad_range = false, bad_order = false;
+#pragma unroll
+    for (int it = 0; it < kHistItems; ++it) {
+        const long i = base + (long)it * kHistThreads + threadIdx.x;
+        if (i >= n) continue;
+        if ((unsigned)v[it] >= (unsigned)U) {
+            bad_range = true;
+        } else {
+            atomicAdd(&h[v[it] >> low_bits], 1);
+        }
+        // neighbour in memory = the next thread's element of the same round
+        int nb = __shfl_down(v[it], 1, 64);
+        if ((threadIdx.x & 63) == 63) nb = (i + 1 < n) ? inv[i + 1] : 0x7fffffff;
+        if (i + 1 < n && nb < v[it]) bad_order = true;
+    }
+    const int f = (__ballot(bad_order) != 0ull ? kFlagUnsorted : 0) | (__ballot(bad_range) != 0ull ? kFlagOutOfRange : 0);
+    if (f && (threadIdx.x & 63) == 0) atomicOr(&s_flags, f);
+    __syncthreads();
+    for (int d = threadIdx.x; d < high_bins; d += kHistThreads) hist[(long)d * n_tiles + blockIdx.x] = h[d];
+    if (threadIdx.x == 0) tile_flags[blockIdx.x] = s_flags;
+}
+
+// id at position i: of unq_inv itself (rows in order) or of the (id, row) pairs the bucket scatter wrote
+__device__ __forceinline__ int kread(const int *keys, long i, bool packed) {
+    return packed ? keys[2 * i] : keys[i];
+}
+
+// Stable scatter by the high digit.  hist: the exclusive scan of the digit-major tile histograms.
+//   bucket_start [high_bins + 1] (written by workgroup 0): first position of every bucket.
+//   stats: zero-filled here (workgroup 0), then UNSORTED / OUT_OF_RANGE of the whole input
+//   and NEED_GENERAL (a bucket above `giant` rows: the bucket kernels step aside).
+// Rows already in order are not moved: out_keys (if given) receives a copy of the ids, and
+// the next kernel reads unq_inv itself.  out_pairs: (id, row) per position, one 8-byte
+// store; or out_keys / out_rows as two arrays when the order is already final.
+__global__ __launch_bounds__(kHistThreads) void bucket_scatter_kernel(
+    const int *__restrict__ inv, long n, int U, int low_bits, int high_bits,
+    const int *__restrict__ hist, const int *__restrict__ tile_flags, int n_tiles, long giant,
+    int *__restrict__ bucket_start, int *__restrict__ stats, int *__restrict__ out_keys,
+    int *__restrict__ out_rows, int2 *__restrict__ out_pairs) {
+    extern __shared__ int wcount[];  // [kHistWaves][bins], then base[bins]
+    __shared__ int s_flags;
+    const int bins = 1 << high_bits;
+    int *base_s = wcount + kHistWaves * bins;  // first destination of this tile's rows, per digit
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const unsigned long long lanes_below = (1ull << lane) - 1ull;
+    if (threadIdx.x == 0) s_flags = 0;
+    for (int k = threadIdx.x; k < kHistWaves * bins; k += kHistThreads) wcount[k] = 0;
+    __syncthreads();
+
+    // ---- flags of the whole input
+    int f = 0;
+    for (int t = threadIdx.x; t < n_tiles; t += kHistThreads) f |= tile_flags[t];
+    if (f) atomicOr(&s_flags, f);
+
+    // ---- first destination of this tile's rows per digit (from the scanned histogram), the
+    // bucket boundaries (workgroup 0 publishes them) and the test for an overfull bucket
+    for (int d = threadIdx.x; d < bins; d += kHistThreads) {
+        const int first = hist[(long)d * n_tiles];
+        const int next = hist[(long)(d + 1) * n_tiles];  // the entry after the last bucket holds the total
+        base_s[d] = hist[(long)d * n_tiles + blockIdx.x];
+        if (blockIdx.x == 0) {
+            bucket_start[d] = first;
+            if (d == bins - 1) bucket_start[bins] = next;
+        }
+        if ((long)next - first > giant) atomicOr(&s_flags, 4);
+    }
+    __syncthreads();
+    const int flags = s_flags;
+    if (blockIdx.x == 0) {
+        for (int k = threadIdx.x; k < TXS_STATS_LEN; k += kHistThreads) {
+            int val = 0;
+            if (k == TXS_STAT_UNSORTED) val = (flags & kFlagUnsorted) ? 1 : 0;
+            if (k == TXS_STAT_OUT_OF_RANGE) val = (flags & kFlagOutOfRange) ? 1 : 0;
+            if (k == TXS_STAT_NEED_GENERAL) val = (flags & 4) ? 1 : 0;
+            stats[k] = val;
+        }
+    }
+    if (flags & 4) return;  // the caller re-plans with the general sequence
+    const long tile0 = (long)blockIdx.x * kHistTile;
+    if (!(flags & kFlagUnsorted)) {
+        if (out_keys)
+            for (int it = 0; it < kHistItems; ++it) {
+                const long i = tile0 + (long)it * kHistThreads + threadIdx.x;
+                if (i < n) out_keys[i] = inv[i];
+            }
+        return;
+    }
+
+    // ---- stable ranking inside the tile and the scatter
+    const long wbase = tile0 + (long)w * (64 * kHistItems);
+    int key[kHistItems], lrank[kHistItems];
+#pragma unroll
+    for (int it = 0; it < kHistItems; ++it) {
+        const long i = wbase + (long)it * 64 + lane;
+        const int v = i < n ? inv[i] : -1;
+        key[it] = (unsigned)v < (unsigned)U ? v : -1;  // out-of-range ids are dropped (and flagged)
+    }
+    volatile int *wc = wcount + w * bins;
+#pragma unroll
+    for (int it = 0; it < kHistItems; ++it) {
+        const bool valid = key[it] >= 0;
+        const int digit = valid ? (key[it] >> low_bits) : 0;
+        unsigned long long mask = __ballot(valid);
+        for (int b = 0; b < high_bits; ++b) {
+            const bool bit = (digit >> b) & 1;
+            const unsigned long long bal = __ballot(bit);
+            mask &= bit ? bal : ~bal;
+        }
+        const int below = __popcll(mask & lanes_below);
+        const int prev = wc[digit];
+        __builtin_amdgcn_wave_barrier();
+        if (valid && below == 0) wc[digit] = prev + __popcll(mask);
+        __builtin_amdgcn_wave_barrier();
+        lrank[it] = prev + below;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < kHistItems; ++it) {
+        if (key[it] < 0) continue;
+        const long i = wbase + (long)it * 64 + lane;
+        const int dg = key[it] >> low_bits;
+        int before = base_s[dg];
+        for (int k = 0; k < w; ++k) before += wcount[k * bins + dg];
+        const long dst = (long)before + lrank[it];
+        if (dst >= 0 && dst < n) {
+            if (out_pairs) {
+                out_pairs[dst] = make_int2(key[it], (int)i);
+            } else {
+                out_keys[dst] = key[it];
+                out_rows[dst] = (int)i;
+            }
+        }
+    }
+}
+
+// Workgroup g serves slice j of bucket b; (b, j) follows from the bucket sizes.
+__global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
+    const int *__restrict__ inv, const int *__restrict__ pairs1, long n, int U,
+    int low_bits, int high_bins, const int *__restrict__ bucket_start, int heavy_threshold,
+    const long long *__restrict__ unq_cnts, int *__restrict__ perm, int *__restrict__ seg,
+    int *__restrict__ preSum, int *__restrict__ slot_of, int *__restrict__ heavy_ids,
+    int *__restrict__ stats) {
+    extern __shared__ int wc[];  // [kBktWaves][low_bins], tot[low_bins], off[low_bins]
+    __shared__ int s_pick[2], s_red[kBktWaves], s_bad[kBktWaves];
+    const int low_bins = 1 << low_bits;
+    int *tot = wc + kBktWaves * low_bins;
+    int *off = tot + low_bins;
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const unsigned long long lanes_below = (1ull << lane) - 1ull;
+    if (stats[TXS_STAT_NEED_GENERAL] != 0) return;
+
+    // ---- which (bucket, slice) is this workgroup's?
+    {
+        if (threadIdx.x == 0) s_pick[0] = -1;
+        int carried = 0;
+        for (int bb0 = 0; bb0 < high_bins; bb0 += kThreads) {
+            const int bb = bb0 + (int)threadIdx.x;
+            int nsl = 0;
+            if (bb < high_bins && ((long)bb << low_bits) < (long)U) {
+                const long cnt_b = (long)bucket_start[bb + 1] - bucket_start[bb];
+                nsl = (int)min((long)kBktMaxSlices, max(1L, (cnt_b + kBktSlice - 1) / kBktSlice));
+            }
+            int total;
+            const int first = carried + block_exclusive_scan(nsl, &total);  // (synchronises the workgroup)
+            if ((int)blockIdx.x >= first && (int)blockIdx.x < first + nsl) {
+                s_pick[0] = bb;
+                s_pick[1] = (int)blockIdx.x - first;
+            }
+            carried += total;
+        }
+        __syncthreads();
+    }
+    const int b = s_pick[0], j = s_pick[1];
+    if (b < 0) return;
+    const int u_lo = b << low_bits;
+    const int u_hi = min(U, u_lo + low_bins);
+    const bool unsorted = stats[TXS_STAT_UNSORTED] != 0;
+    const bool packed = unsorted;
+    const int *keys = unsorted ? pairs1 : inv;
+    const long s = bucket_start[b];
+    const long e = bucket_start[b + 1];
+    const long nb = e - s;
+    long slice = kBktSlice;
+    if (nb > (long)kBktMaxSlices * kBktSlice)
+        slice = ((nb + kBktMaxSlices - 1) / kBktMaxSlices + kBktChunk - 1) / kBktChunk * kBktChunk;
+    const long my_s = s + (long)j * slice;
+    const long my_e = min(e, my_s + slice);
+
+    // ---- counts of the bucket's voxels, and of the rows in front of this slice
+    for (int k = threadIdx.x; k < (kBktWaves + 2) * low_bins; k += kThreads) wc[k] = 0;
+    __syncthreads();
+    for (long i0 = s; i0 < e; i0 += (long)kThreads * kBktItems) {
+        int v[kBktItems];  // all loads of a round in flight before the first count
+#pragma unroll
+        for (int it = 0; it < kBktItems; ++it) {
+            const long i = i0 + (long)it * kThreads + threadIdx.x;
+            v[it] = i < e ? kread(keys, i, packed) : -1;
+        }
+#pragma unroll
+        for (int it = 0; it < kBktItems; ++it) {
+            const long i = i0 + (long)it * kThreads + threadIdx.x;
+            const int d = v[it] - u_lo;
+            if (i < e && (unsigned)d < (unsigned)low_bins) {
+                atomicAdd(&tot[d], 1);
+                if (i < my_s) atomicAdd(&off[d], 1);
+            }
+        }
+    }
+    __syncthreads();
+    // ---- exclusive scan over the voxels of the bucket: a run of consecutive voxels per thread
+    const int per = (low_bins + kThreads - 1) / kThreads;
+    const int d0 = threadIdx.x * per;
+    int mine = 0;
+    for (int k = 0; k < per; ++k)
+        if (d0 + k < low_bins) mine += tot[d0 + k];
+    int total;
+    int run = block_exclusive_scan(mine, &total);
+    // off[d] becomes the bucket-relative position of the slice's first row of voxel d
+    for (int k = 0; k < per; ++k) {
+        const int d = d0 + k;
+        if (d >= low_bins) break;
+        const int c = tot[d];
+        const int excl = run;
+        run += c;
+        off[d] += excl;
+        if (j == 0 && u_lo + d < u_hi) {
+            preSum[u_lo + d] = (int)s + excl;
+            if (u_lo + d == U - 1) preSum[U] = (int)n;
+        }
+    }
+    __syncthreads();
+    // ---- statistics, special voxels and their slots (first slice only; as plan_special_kernel)
+    if (j == 0) {
+        int vmax = 0;
+        bool mismatch = false;
+        for (int dd = 0; dd < low_bins; dd += kThreads) {
+            const int d = dd + (int)threadIdx.x;
+            const int u = u_lo + d;
+            const bool in = d < low_bins && u < u_hi;
+            const int cnt = in ? tot[d] : 0;
+            vmax = max(vmax, cnt);
+            mismatch |= in && unq_cnts && unq_cnts[u] != (long long)cnt;
+            const bool heavy = in && cnt > heavy_threshold;
+            const bool empty = in && cnt == 0;
+            const unsigned long long mh = __ballot(heavy), me = __ballot(empty);
+            int base_h = 0, base_e = 0;
+            if (lane == 0) {
+                if (mh) base_h = atomicAdd(&stats[TXS_STAT_NUM_HEAVY], __popcll(mh));
+                if (me) base_e = atomicAdd(&stats[TXS_STAT_NUM_EMPTY], __popcll(me));
+                if (mh | me) atomicAdd(&stats[TXS_STAT_NUM_SPECIAL], __popcll(mh) + __popcll(me));
+            }
+            base_h = __shfl(base_h, 0, 64);
+            base_e = __shfl(base_e, 0, 64);
+            if (in) {
+                int slot = -1;
+                if (heavy) {
+                    slot = base_h + __popcll(mh & lanes_below);
+                    if (slot < U) heavy_ids[slot] = u;
+                } else if (empty) {
+                    slot = U - 1 - (base_e + __popcll(me & lanes_below));
+                    if (slot >= 0) heavy_ids[slot] = u;
+                }
+                slot_of[u] = slot;
+            }
+        }
+        const int wmax = wave_max_i32(vmax);
+        const bool any_mismatch = __ballot(mismatch) != 0ull;
+        if (lane == 0) {
+            s_red[w] = wmax;
+            s_bad[w] = any_mismatch;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int m = 0, bad = 0;
+            for (int k = 0; k < kBktWaves; ++k) {
+                m = max(m, s_red[k]);
+                bad |= s_bad[k];
+            }
+            if (m > 0) atomicMax(&stats[TXS_STAT_MAX_CNT], m);
+            if (bad) stats[TXS_STAT_COUNT_MISMATCH] = 1;
+        }
+    }
+
+    // ---- stable placement of the slice by the low digit, round after round
+    for (long c0 = my_s; c0 < my_e; c0 += kBktChunk) {
+        int key[kBktItems], row[kBktItems], lrank[kBktItems];
+        volatile int *mywc = wc + w * low_bins;
+        const long wbase = c0 + (long)w * (64 * kBktItems);
+#pragma unroll
+        for (int it = 0; it < kBktItems; ++it) {
+            const long i = wbase + (long)it * 64 + lane;
+            int v = -1;
+            row[it] = (int)i;
+            if (i < my_e) {
+                if (packed) {
+                    const int2 kr = reinterpret_cast<const int2 *>(pairs1)[i];
+                    v = kr.x;
+                    row[it] = kr.y;
+                } else {
+                    v = inv[i];
+                }
+            }
+            key[it] = (i < my_e && (unsigned)(v - u_lo) < (unsigned)low_bins) ? v : -1;
+        }
+#pragma unroll
+        for (int it = 0; it < kBktItems; ++it) {
+            const bool valid = key[it] >= 0;
+            const int digit = valid ? key[it] - u_lo : 0;
+            unsigned long long mask = __ballot(valid);
+            for (int bb = 0; bb < low_bits; ++bb) {
+                const bool bit = (digit >> bb) & 1;
+                const unsigned long long bal = __ballot(bit);
+                mask &= bit ? bal : ~bal;
+            }
+            const int below = __popcll(mask & lanes_below);
+            const int prev = mywc[digit];
+            __builtin_amdgcn_wave_barrier();
+            if (valid && below == 0) mywc[digit] = prev + __popcll(mask);
+            __builtin_amdgcn_wave_barrier();
+            lrank[it] = prev + below;
+        }
+        __syncthreads();
+        // destination = slice-start position of the voxel + rows of the voxel that the waves
+        // in front of this one hold in this round + rank inside the wave; the per-voxel
+        // bookkeeping is done per ROW (a few LDS operations each), never per voxel: a round
+        // has fewer rows than a bucket can have voxel-times-wave counters
+        long dst[kBktItems];
+#pragma unroll
+        for (int it = 0; it < kBktItems; ++it) {
+            dst[it] = -1;
+            if (key[it] < 0) continue;
+            const int dg = key[it] - u_lo;
+            int before = off[dg];
+            for (int k = 0; k < w; ++k) before += wc[k * low_bins + dg];
+            dst[it] = s + before + lrank[it];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < kBktItems; ++it) {
+            if (key[it] < 0) continue;
+            const int dg = key[it] - u_lo;
+            atomicAdd(&off[dg], 1);       // the next round starts behind this round's rows
+            wc[w * low_bins + dg] = 0;    // (every row of the group stores the same zero)
+            if (dst[it] >= s && dst[it] < e) {
+                const int c = tot[dg];
+                seg[dst[it]] = key[it] | (c > heavy_threshold ? kSpecialBit : 0);
+                if (unsorted) perm[dst[it]] = row[it];
+            }
+        }
+        __syncthreads();
+    }
+}
+
 int radix_bits(int64_t U) {
     int bits = 1;
     while ((1LL << bits) < U) ++bits;
@@ -449,6 +854,106 @@ int txs_plan_seg_from_presum(const int32_t *preSum, int64_t num_total, int64_t n
     if (!preSum || !slot_of || !seg || num_unq <= 0) return TXS_ERR_INVALID_ARG;
     seg_from_presum_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
         preSum, num_total, (int)num_unq, slot_of, seg);
+    return status_of(hipGetLastError());
+}
+
+int64_t txs_plan_workspace_len(int64_t num_total, int64_t num_unq) {
+    if (!fits_i32(num_total) || !fits_i32(num_unq)) return -1;
+    const int64_t general = txs_sort_workspace_len(num_total, num_unq);
+    const int64_t tiles = (num_total + kHistTile - 1) / kHistTile;
+    const int64_t bins = (int64_t)1 << kBucketLowBitsMax;
+    // (id, row) pairs after the bucket scatter, the digit-major histogram, tile flags, bucket
+    // boundaries, the scan workspace
+    const int64_t hist = bins * (tiles > 0 ? tiles : 1) + 1;
+    const int64_t bucket = 2 * num_total + hist + tiles + bins + 1 + scan_tiles(hist + 1) + 17;
+    return general > bucket ? general : bucket;
+}
+
+int txs_plan_build_general(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, int32_t heavy_threshold,
+                           const int64_t *unq_cnts, int32_t *plan_ws, int32_t *perm, int32_t *seg,
+                           int32_t *preSum, int32_t *slot_of, int32_t *heavy_ids, int32_t *stats, void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_unq) || !stats || !preSum || heavy_threshold < kChunk)
+        return TXS_ERR_INVALID_ARG;
+    const long n = num_total;
+    const int U = (int)num_unq;
+    if (n > 0 && (!unq_inv || !plan_ws || !perm || !seg)) return TXS_ERR_INVALID_ARG;
+    if (U > 0 && (!slot_of || !heavy_ids)) return TXS_ERR_INVALID_ARG;
+    // order/range flags, three-kernel radix passes, CSR offsets, special table, flags
+    int rc = txs_plan_check(unq_inv, n, U, stats, stream);
+    if (rc == TXS_OK && n > 0 && U > 0) rc = txs_plan_sort(unq_inv, n, U, stats, perm, seg, plan_ws, stream);
+    if (rc == TXS_OK) rc = txs_plan_presum(seg, U > 0 ? n : 0, U, preSum, stream);
+    if (rc == TXS_OK)
+        rc = txs_plan_special(preSum, U, heavy_threshold, unq_cnts, slot_of, heavy_ids, stats, nullptr, nullptr,
+                              stream);
+    if (rc == TXS_OK) rc = txs_plan_seg_flag(seg, U > 0 ? n : 0, U, slot_of, stream);
+    return rc;
+}
+
+int txs_plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, int32_t heavy_threshold,
+                   const int64_t *unq_cnts, int32_t *plan_ws, int32_t *perm, int32_t *seg, int32_t *preSum,
+                   int32_t *slot_of, int32_t *heavy_ids, int32_t *stats, void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_unq) || !stats || !preSum || heavy_threshold < kChunk)
+        return TXS_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const long n = num_total;
+    const int U = (int)num_unq;
+    if (n > 0 && (!unq_inv || !plan_ws || !perm || !seg)) return TXS_ERR_INVALID_ARG;
+    if (U > 0 && (!slot_of || !heavy_ids)) return TXS_ERR_INVALID_ARG;
+    if (((uintptr_t)plan_ws & 7u) != 0) return TXS_ERR_INVALID_ARG;
+    const int bits = radix_bits(U > 1 ? U : 1);
+    if (n == 0 || U == 0 || bits > kBucketBitsMax)
+        return txs_plan_build_general(unq_inv, num_total, num_unq, heavy_threshold, unq_cnts, plan_ws, perm, seg,
+                                      preSum, slot_of, heavy_ids, stats, stream);
+    // ids of up to 11 bits are sorted by the bucket pass alone; beyond that the bucket digit has
+    // 8 bits (a tile then sends runs of about 32 rows to every bucket and the scatter writes
+    // whole cache lines) and the low digit takes the rest, at most 11
+    const int low_bits = bits <= kBucketLowBitsMax ? 0 : min(bits - kBucketHighBits, kBucketLowBitsMax);
+    const int high_bits = bits - low_bits;
+    const int high_bins = 1 << high_bits;
+    const int n_tiles = (int)((n + kHistTile - 1) / kHistTile);
+    int *pairs1 = plan_ws;  // (id, row) after the bucket scatter, 8-byte aligned
+    int *hist = plan_ws + 2 * n;
+    const long used = (long)high_bins * n_tiles;
+    int *tile_flags = hist + used + 1;
+    int *bucket_start = tile_flags + n_tiles;
+    int *scan_ws = bucket_start + high_bins + 1;
+    static bool lds_allowed = false;
+    if (!lds_allowed) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(bucket_scatter_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) != hipSuccess)
+            return TXS_ERR_LAUNCH;
+        lds_allowed = true;
+    }
+    bucket_hist_kernel<<<dim3(n_tiles), dim3(kHistThreads), 0, st>>>(unq_inv, n, U, low_bits, high_bins, hist,
+                                                                     tile_flags, n_tiles);
+    // one entry more than the histogram: it receives the total, the end of the last bucket
+    if (exclusive_scan(hist, used, hist, used + 1, scan_ws, st) != hipSuccess) return TXS_ERR_LAUNCH;
+    const size_t lds_scatter = (size_t)(kHistWaves + 1) * high_bins * sizeof(int);
+    if (low_bits == 0) {
+        // a bucket is a voxel: the scatter already gives the final order
+        bucket_scatter_kernel<<<dim3(n_tiles), dim3(kHistThreads), lds_scatter, st>>>(
+            unq_inv, n, U, low_bits, high_bits, hist, tile_flags, n_tiles, n + 1, bucket_start, stats, seg, perm,
+            nullptr);
+        int rc = txs_plan_presum(seg, n, U, preSum, stream);
+        if (rc == TXS_OK)
+            rc = txs_plan_special(preSum, U, heavy_threshold, unq_cnts, slot_of, heavy_ids, stats, nullptr, nullptr,
+                                  stream);
+        if (rc == TXS_OK) rc = txs_plan_seg_flag(seg, n, U, slot_of, stream);
+        return rc;
+    }
+    // a bucket so full that its workgroups would run long after all others have finished
+    // (only a few voxels holding most of the rows do that) sends the call to the general sequence
+    const long giant = (long)kBktMaxSlices * kBktSlice * 2;
+    bucket_scatter_kernel<<<dim3(n_tiles), dim3(kHistThreads), lds_scatter, st>>>(
+        unq_inv, n, U, low_bits, high_bits, hist, tile_flags, n_tiles, giant, bucket_start, stats, nullptr,
+        nullptr, reinterpret_cast<int2 *>(pairs1));
+    const int low_bins = 1 << low_bits;
+    const size_t lds = (size_t)(kBktWaves + 2) * low_bins * sizeof(int);
+    // an upper bound of the (bucket, slice) pairs; workgroups beyond the last pair return at once
+    const long groups = n / kBktSlice + high_bins;
+    bucket_plan_kernel<<<dim3((unsigned)groups), dim3(kThreads), lds, st>>>(
+        unq_inv, pairs1, n, U, low_bits, high_bins, bucket_start, heavy_threshold,
+        (const long long *)unq_cnts, perm, seg, preSum, slot_of, heavy_ids, stats);
     return status_of(hipGetLastError());
 }
 

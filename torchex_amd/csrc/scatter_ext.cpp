@@ -67,7 +67,11 @@ Tensor empty_i32(int64_t n, const Tensor &like) {
 }
 
 std::vector<int64_t> read_stats(const Tensor &stats) {
-    Tensor h = stats.cpu();  // the one host synchronisation of index preparation
+    // the one host synchronisation of index preparation: an asynchronous copy into pinned
+    // host memory (from the caching host allocator), then a wait on the stream
+    Tensor h = at::empty({TXS_STATS_LEN}, stats.options().device(at::kCPU).pinned_memory(true));
+    h.copy_(stats, /*non_blocking=*/true);
+    c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(stats.device().index()).synchronize();
     std::vector<int64_t> v(TXS_STATS_LEN);
     for (int i = 0; i < TXS_STATS_LEN; ++i) v[i] = h.data_ptr<int32_t>()[i];
     return v;
@@ -110,23 +114,34 @@ std::tuple<Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>> buil
     Tensor preSum = empty_i32(U + 1, unq_inv);
     Tensor slot_of = empty_i32(U, unq_inv);
     Tensor heavy_all = empty_i32(U, unq_inv);
-    check_status(txs_plan_check(i32p(unq_inv), N, U, i32w(stats), st), "plan_check");
+    std::vector<int64_t> hs;
     if (assume_sorted) {
+        check_status(txs_plan_check(i32p(unq_inv), N, U, i32w(stats), st), "plan_check");
         seg = unq_inv.clone();  // sorted ids are their own sorted keys
+        check_status(txs_plan_presum(i32p(seg), U > 0 ? N : 0, U, i32w(preSum), st), "plan_presum");
+        check_status(txs_plan_special(i32p(preSum), U, (int32_t)heavy_threshold, cnts, i32w(slot_of),
+                                      i32w(heavy_all), i32w(stats), nullptr, nullptr, st),
+                     "plan_special");
+        check_status(txs_plan_seg_flag(i32w(seg), U > 0 ? N : 0, U, i32p(slot_of), st), "plan_seg_flag");
+        hs = read_stats(stats);
     } else {
         seg = empty_i32(N, unq_inv);
         perm = empty_i32(N, unq_inv);
-        Tensor ws = empty_i32(txs_sort_workspace_len(N, U), unq_inv);
-        if (U > 0)
-            check_status(txs_plan_sort(i32p(unq_inv), N, U, i32p(stats), i32w(perm), i32w(seg), i32w(ws), st),
-                         "plan_sort");
+        Tensor ws = empty_i32(txs_plan_workspace_len(N, U), unq_inv);
+        check_status(txs_plan_build(i32p(unq_inv), N, U, (int32_t)heavy_threshold, cnts, i32w(ws), i32w(perm),
+                                    i32w(seg), i32w(preSum), i32w(slot_of), i32w(heavy_all), i32w(stats), st),
+                     "plan_build");
+        hs = read_stats(stats);
+        if (hs[TXS_STAT_NEED_GENERAL]) {
+            // a few voxels own most of the rows: the bucket kernels stepped aside
+            stats.zero_();
+            check_status(txs_plan_build_general(i32p(unq_inv), N, U, (int32_t)heavy_threshold, cnts, i32w(ws),
+                                                i32w(perm), i32w(seg), i32w(preSum), i32w(slot_of),
+                                                i32w(heavy_all), i32w(stats), st),
+                         "plan_build_general");
+            hs = read_stats(stats);
+        }
     }
-    check_status(txs_plan_presum(i32p(seg), U > 0 ? N : 0, U, i32w(preSum), st), "plan_presum");
-    check_status(txs_plan_special(i32p(preSum), U, (int32_t)heavy_threshold, cnts, i32w(slot_of),
-                                  i32w(heavy_all), i32w(stats), nullptr, nullptr, st),
-                 "plan_special");
-    check_status(txs_plan_seg_flag(i32w(seg), U > 0 ? N : 0, U, i32p(slot_of), st), "plan_seg_flag");
-    std::vector<int64_t> hs = read_stats(stats);
     TORCH_CHECK(hs[TXS_STAT_OUT_OF_RANGE] == 0 && (U > 0 || N == 0),
                 "unq_inv holds ids outside [0, num_unq=", U, ")");
     TORCH_CHECK(!(assume_sorted && hs[TXS_STAT_UNSORTED]),
