@@ -280,6 +280,30 @@ def test_grid_hash_build_and_probe_against_oracle():
         assert np.array_equal(orc.grid_hash_probe(queries, tb), out)
 
 
+def test_grid_hash_absent_keys():
+    """Keys that are not in the table.  With free slots in the table (N not a power of two)
+    the probe of an absent key stops at the first empty slot of its sequence, so 200k of them
+    cost about as much as 200k present ones.  On a completely full table (N a power of two,
+    the table has exactly N slots as in the reference, grid_hash.cpp:28-37) there is no empty
+    slot and an absent key is looked for in all N slots -- the reference does that for every
+    absent key on any table (functions.cuh:54-63) -- so only 32 are asked for here:
+    32 x 262,144 slot reads."""
+    T = tx()
+    rng = np.random.default_rng(23)
+    for n, n_absent in ((300_000, 200_000), (1 << 18, 32)):
+        keys = rng.choice(2 ** 30, size=n, replace=False).astype(np.int32)
+        vals = rng.permutation(n).astype(np.int32)
+        absent = np.setdiff1d(rng.integers(0, 2 ** 30, size=n_absent + 64).astype(np.int32), keys)[:n_absent]
+        queries = np.concatenate([absent, keys[:1000]])
+        want = np.concatenate([np.full(absent.shape[0], -1, np.int32), vals[:1000]])
+        table = T.grid_hash_build(torch.from_numpy(keys).to(DEV), torch.from_numpy(vals).to(DEV))
+        free = int((table[:, 0] == -1).sum())
+        say(f"[case] grid_hash absent keys n={n} table={table.shape[0]} free={free} absent={absent.shape[0]}")
+        assert (free == 0) == ((n & (n - 1)) == 0)
+        out = T.grid_hash_probe(torch.from_numpy(queries).to(DEV), table).cpu().numpy()
+        assert np.array_equal(out, want)
+
+
 def test_grid_hash_class_follows_the_reference_test():
     """test/test_grid_hash.py:17-44 (smaller, seeded): probe(unique rows) == arange, the
     table maps its own keys to their values, and the mapping is stable under re-indexing."""
