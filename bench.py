@@ -260,13 +260,14 @@ def measure(T, scatter_ext, workloads, names, w, dtype, steps, warmup, dev, extr
     inv, cnts = w.unq_inv.to(dev), w.unq_cnts.to(dev)
     g_mean, g_max = g_mean_cpu.to(dev).to(tdt), g_max_cpu.to(dev).to(tdt)
 
-    data = T.ScatterData(inv, cnts)        # index preparation, timed separately
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(5):
+    for _ in range(3):                     # index preparation, timed separately
         data = T.ScatterData(inv, cnts)
     torch.cuda.synchronize()
-    prep_ms = (time.perf_counter() - t0) / 5 * 1e3
+    t0 = time.perf_counter()
+    for _ in range(20):
+        data = T.ScatterData(inv, cnts)
+    torch.cuda.synchronize()
+    prep_ms = (time.perf_counter() - t0) / 20 * 1e3
 
     def step():
         feats.grad = None
@@ -304,7 +305,6 @@ def measure(T, scatter_ext, workloads, names, w, dtype, steps, warmup, dev, extr
         kt["sum_fwd"] = event_ms(lambda: scatter_ext.forward(scatter_ext.SUM, f, *plan), it)
         kt["sum_bwd"] = event_ms(lambda: scatter_ext.backward(scatter_ext.SUM, g_mean, None, *bplan), it)
         kt["max_reftie_fwd"] = event_ms(lambda: scatter_ext.forward(scatter_ext.MAX_REFTIE, f, *plan), it)
-        res["max_fwd_back_to_back_ms"] = event_ms(lambda: scatter_ext.forward(scatter_ext.MAX, f, *plan), it)
     ab = {k: workloads.algorithmic_bytes(k.replace("max_reftie", "max"), N, C, U, esz) for k in kt}
     res["kt"] = kt
     res["ab"] = ab
@@ -436,7 +436,6 @@ def main():
         "per_op": r["per_op"],
         "per_kernel": per_kernel,
         "kernel_sum_ms": r["kernel_sum_ms"],
-        "max_fwd_back_to_back_ms": r["max_fwd_back_to_back_ms"],
         "sorted_input": sorted_input,
         "device_copy_GBps": copy_gbps,
         "index_prep_ms": r["prep_ms"],
