@@ -51,7 +51,8 @@ OTHER_CONFIGS = (("uniform_box", "f32"), ("lidar_sweep", "f16"), ("lidar_sweep",
 # (workload, dtype, kernel), together with a digest of the kernel sources they were
 # measured on: figures are reported only while the sources still match.
 TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_table.json")
-KERNEL_SOURCES = ("torchex_amd/csrc/scatter_kernels.hip", "torchex_amd/csrc/txs_common.h")
+KERNEL_SOURCES = ("torchex_amd/csrc/scatter_kernels.hip", "torchex_amd/csrc/table_kernels.hip",
+                  "torchex_amd/csrc/txs_common.h")
 
 
 def parse():
