@@ -358,20 +358,35 @@ __global__ void seg_from_presum_kernel(const int *__restrict__ preSum, long n, i
 // costs more than it saves from about 100 tiles on; per-voxel instead of per-row offset
 // bookkeeping in (4) makes no difference.
 
-constexpr int kBucketHighBits = 8;
+#ifndef TXS_BUCKET_HIGH_BITS
+#define TXS_BUCKET_HIGH_BITS 9
+#endif
+constexpr int kBucketHighBits = TXS_BUCKET_HIGH_BITS;
 constexpr int kBucketLowBitsMax = 11;   // also the largest high digit
 constexpr int kBucketBitsMax = 22;
-constexpr int kHistThreads = 512, kHistItems = 16;
-constexpr int kHistTile = kHistThreads * kHistItems;  // 8192 rows per tile
+constexpr int kHistThreads = 512;
+// rows per tile of the histogram and scatter kernels: 512 * {4, 8, 16}, the largest that still
+// gives every compute unit a tile
+int hist_items_for(long n) {
+    return n >= 256L * kHistThreads * 16 ? 16 : (n >= 256L * kHistThreads * 8 ? 8 : 4);
+}
 constexpr int kHistWaves = kHistThreads / 64;
-constexpr int kBktItems = 16;
+#ifndef TXS_BKT_ITEMS
+#define TXS_BKT_ITEMS 8
+#endif
+#ifndef TXS_BKT_SLICE_CHUNKS
+#define TXS_BKT_SLICE_CHUNKS 1
+#endif
+constexpr int kBktItems = TXS_BKT_ITEMS;
 constexpr int kBktChunk = kThreads * kBktItems;        // 4096 rows per placement round
 constexpr int kBktWaves = kThreads / 64;
-constexpr int kBktSlice = 2 * kBktChunk;               // rows one workgroup places
+constexpr int kBktSlice = TXS_BKT_SLICE_CHUNKS * kBktChunk;  // rows one workgroup places
 constexpr int kBktMaxSlices = 16;                      // workgroups per bucket at most
+constexpr long kBktGiant = 262144;                     // rows in one bucket beyond which the general sequence runs
 constexpr int kFlagUnsorted = 1, kFlagOutOfRange = 2;
 
 // hist: [high_bins][n_tiles] digit-major (the order its exclusive scan needs); tile_flags: [n_tiles]
+template <int ITEMS>
 __global__ __launch_bounds__(kHistThreads) void bucket_hist_kernel(
     const int *__restrict__ inv, long n, int U, int low_bits, int high_bins, int *__restrict__ hist,
     int *__restrict__ tile_flags, int n_tiles) {
@@ -380,16 +395,16 @@ __global__ __launch_bounds__(kHistThreads) void bucket_hist_kernel(
     for (int d = threadIdx.x; d < high_bins; d += kHistThreads) h[d] = 0;
     if (threadIdx.x == 0) s_flags = 0;
     __syncthreads();
-    const long base = (long)blockIdx.x * kHistTile;
-    int v[kHistItems];
+    const long base = (long)blockIdx.x * (kHistThreads * ITEMS);
+    int v[ITEMS];
 #pragma unroll
-    for (int it = 0; it < kHistItems; ++it) {
+    for (int it = 0; it < ITEMS; ++it) {
         const long i = base + (long)it * kHistThreads + threadIdx.x;
         v[it] = i < n ? inv[i] : 0x7fffffff;
     }
     bool bad_range = false, bad_order = false;
 #pragma unroll
-    for (int it = 0; it < kHistItems; ++it) {
+    for (int it = 0; it < ITEMS; ++it) {
         const long i = base + (long)it * kHistThreads + threadIdx.x;
         if (i >= n) continue;
         if ((unsigned)v[it] >= (unsigned)U) {
@@ -421,6 +436,7 @@ __device__ __forceinline__ int kread(const int *keys, long i, bool packed) {
 // Rows already in order are not moved: out_keys (if given) receives a copy of the ids, and
 // the next kernel reads unq_inv itself.  out_pairs: (id, row) per position, one 8-byte
 // store; or out_keys / out_rows as two arrays when the order is already final.
+template <int ITEMS>
 __global__ __launch_bounds__(kHistThreads) void bucket_scatter_kernel(
     const int *__restrict__ inv, long n, int U, int low_bits, int high_bits,
     const int *__restrict__ hist, const int *__restrict__ tile_flags, int n_tiles, long giant,
@@ -465,10 +481,10 @@ __global__ __launch_bounds__(kHistThreads) void bucket_scatter_kernel(
         }
     }
     if (flags & 4) return;  // the caller re-plans with the general sequence
-    const long tile0 = (long)blockIdx.x * kHistTile;
+    const long tile0 = (long)blockIdx.x * (kHistThreads * ITEMS);
     if (!(flags & kFlagUnsorted)) {
         if (out_keys)
-            for (int it = 0; it < kHistItems; ++it) {
+            for (int it = 0; it < ITEMS; ++it) {
                 const long i = tile0 + (long)it * kHistThreads + threadIdx.x;
                 if (i < n) out_keys[i] = inv[i];
             }
@@ -476,17 +492,17 @@ __global__ __launch_bounds__(kHistThreads) void bucket_scatter_kernel(
     }
 
     // ---- stable ranking inside the tile and the scatter
-    const long wbase = tile0 + (long)w * (64 * kHistItems);
-    int key[kHistItems], lrank[kHistItems];
+    const long wbase = tile0 + (long)w * (64 * ITEMS);
+    int key[ITEMS], lrank[ITEMS];
 #pragma unroll
-    for (int it = 0; it < kHistItems; ++it) {
+    for (int it = 0; it < ITEMS; ++it) {
         const long i = wbase + (long)it * 64 + lane;
         const int v = i < n ? inv[i] : -1;
         key[it] = (unsigned)v < (unsigned)U ? v : -1;  // out-of-range ids are dropped (and flagged)
     }
     volatile int *wc = wcount + w * bins;
 #pragma unroll
-    for (int it = 0; it < kHistItems; ++it) {
+    for (int it = 0; it < ITEMS; ++it) {
         const bool valid = key[it] >= 0;
         const int digit = valid ? (key[it] >> low_bits) : 0;
         unsigned long long mask = __ballot(valid);
@@ -504,7 +520,7 @@ __global__ __launch_bounds__(kHistThreads) void bucket_scatter_kernel(
     }
     __syncthreads();
 #pragma unroll
-    for (int it = 0; it < kHistItems; ++it) {
+    for (int it = 0; it < ITEMS; ++it) {
         if (key[it] < 0) continue;
         const long i = wbase + (long)it * 64 + lane;
         const int dg = key[it] >> low_bits;
@@ -575,24 +591,60 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
     const long my_s = s + (long)j * slice;
     const long my_e = min(e, my_s + slice);
 
+    // the caller's counts of this bucket's voxels (first slice only) are fetched now and
+    // compared once the kernel's own counts are complete
+    constexpr int kCntPer = (1 << kBucketLowBitsMax) / kThreads;
+    long long given[kCntPer];
+    const bool check_counts = j == 0 && unq_cnts != nullptr;
+    if (check_counts) {
+#pragma unroll
+        for (int k = 0; k < kCntPer; ++k) {
+            const int d = k * kThreads + (int)threadIdx.x;
+            given[k] = (d < low_bins && u_lo + d < u_hi) ? unq_cnts[u_lo + d] : -1;
+        }
+    }
     // ---- counts of the bucket's voxels, and of the rows in front of this slice
     for (int k = threadIdx.x; k < (kBktWaves + 2) * low_bins; k += kThreads) wc[k] = 0;
     __syncthreads();
-    for (long i0 = s; i0 < e; i0 += (long)kThreads * kBktItems) {
-        int v[kBktItems];  // all loads of a round in flight before the first count
+    {
+        // two rounds of loads in flight: the next round's ids arrive while this round is counted
+        const long round = (long)kThreads * kBktItems;
+        auto fetch = [&](int (&v)[kBktItems], long i0) {
 #pragma unroll
-        for (int it = 0; it < kBktItems; ++it) {
-            const long i = i0 + (long)it * kThreads + threadIdx.x;
-            v[it] = i < e ? kread(keys, i, packed) : -1;
-        }
-#pragma unroll
-        for (int it = 0; it < kBktItems; ++it) {
-            const long i = i0 + (long)it * kThreads + threadIdx.x;
-            const int d = v[it] - u_lo;
-            if (i < e && (unsigned)d < (unsigned)low_bins) {
-                atomicAdd(&tot[d], 1);
-                if (i < my_s) atomicAdd(&off[d], 1);
+            for (int it = 0; it < kBktItems; ++it) {
+                const long i = i0 + (long)it * kThreads + threadIdx.x;
+                v[it] = i < e ? kread(keys, i, packed) : -1;
             }
+        };
+        auto count = [&](const int (&v)[kBktItems], long i0) {
+#pragma unroll
+            for (int it = 0; it < kBktItems; ++it) {
+                const long i = i0 + (long)it * kThreads + threadIdx.x;
+                const int d = v[it] - u_lo;
+                if (i < e && (unsigned)d < (unsigned)low_bins) {
+                    atomicAdd(&tot[d], 1);
+                    if (i < my_s) atomicAdd(&off[d], 1);
+                }
+            }
+        };
+        int va[kBktItems], vb[kBktItems];
+        long i0 = s;
+        fetch(va, i0);
+        for (;;) {
+            if (i0 + round >= e) {
+                count(va, i0);
+                break;
+            }
+            fetch(vb, i0 + round);
+            count(va, i0);
+            i0 += round;
+            if (i0 + round >= e) {
+                count(vb, i0);
+                break;
+            }
+            fetch(va, i0 + round);
+            count(vb, i0);
+            i0 += round;
         }
     }
     __syncthreads();
@@ -622,13 +674,19 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
     if (j == 0) {
         int vmax = 0;
         bool mismatch = false;
+        if (check_counts) {
+#pragma unroll
+            for (int k = 0; k < kCntPer; ++k) {
+                const int d = k * kThreads + (int)threadIdx.x;
+                if (d < low_bins && u_lo + d < u_hi) mismatch |= given[k] != (long long)tot[d];
+            }
+        }
         for (int dd = 0; dd < low_bins; dd += kThreads) {
             const int d = dd + (int)threadIdx.x;
             const int u = u_lo + d;
             const bool in = d < low_bins && u < u_hi;
             const int cnt = in ? tot[d] : 0;
             vmax = max(vmax, cnt);
-            mismatch |= in && unq_cnts && unq_cnts[u] != (long long)cnt;
             const bool heavy = in && cnt > heavy_threshold;
             const bool empty = in && cnt == 0;
             const unsigned long long mh = __ballot(heavy), me = __ballot(empty);
@@ -860,7 +918,8 @@ int txs_plan_seg_from_presum(const int32_t *preSum, int64_t num_total, int64_t n
 int64_t txs_plan_workspace_len(int64_t num_total, int64_t num_unq) {
     if (!fits_i32(num_total) || !fits_i32(num_unq)) return -1;
     const int64_t general = txs_sort_workspace_len(num_total, num_unq);
-    const int64_t tiles = (num_total + kHistTile - 1) / kHistTile;
+    const int64_t tile = (int64_t)kHistThreads * hist_items_for(num_total);
+    const int64_t tiles = (num_total + tile - 1) / tile;
     const int64_t bins = (int64_t)1 << kBucketLowBitsMax;
     // (id, row) pairs after the bucket scatter, the digit-major histogram, tile flags, bucket
     // boundaries, the scan workspace
@@ -905,12 +964,16 @@ int txs_plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, i
         return txs_plan_build_general(unq_inv, num_total, num_unq, heavy_threshold, unq_cnts, plan_ws, perm, seg,
                                       preSum, slot_of, heavy_ids, stats, stream);
     // ids of up to 11 bits are sorted by the bucket pass alone; beyond that the bucket digit has
-    // 8 bits (a tile then sends runs of about 32 rows to every bucket and the scatter writes
-    // whole cache lines) and the low digit takes the rest, at most 11
+    // 9 bits (narrower, and the buckets of a spatially sorted id space get too uneven: a
+    // bucket's workgroups each count the whole bucket; wider, and a tile sends too few rows to
+    // a bucket for the scatter to write whole cache lines) and the low digit takes the rest,
+    // at most 11
     const int low_bits = bits <= kBucketLowBitsMax ? 0 : min(bits - kBucketHighBits, kBucketLowBitsMax);
     const int high_bits = bits - low_bits;
     const int high_bins = 1 << high_bits;
-    const int n_tiles = (int)((n + kHistTile - 1) / kHistTile);
+    const int items = hist_items_for(n);
+    const long tile = (long)kHistThreads * items;
+    const int n_tiles = (int)((n + tile - 1) / tile);
     int *pairs1 = plan_ws;  // (id, row) after the bucket scatter, 8-byte aligned
     int *hist = plan_ws + 2 * n;
     const long used = (long)high_bins * n_tiles;
@@ -919,19 +982,24 @@ int txs_plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, i
     int *scan_ws = bucket_start + high_bins + 1;
     static bool lds_allowed = false;
     if (!lds_allowed) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(bucket_scatter_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) != hipSuccess)
-            return TXS_ERR_LAUNCH;
+        for (const void *k : {reinterpret_cast<const void *>(bucket_scatter_kernel<4>),
+                              reinterpret_cast<const void *>(bucket_scatter_kernel<8>),
+                              reinterpret_cast<const void *>(bucket_scatter_kernel<16>)})
+            if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) != hipSuccess)
+                return TXS_ERR_LAUNCH;
         lds_allowed = true;
     }
-    bucket_hist_kernel<<<dim3(n_tiles), dim3(kHistThreads), 0, st>>>(unq_inv, n, U, low_bits, high_bins, hist,
-                                                                     tile_flags, n_tiles);
+    auto hist_kernel = items == 16 ? bucket_hist_kernel<16> : (items == 8 ? bucket_hist_kernel<8> : bucket_hist_kernel<4>);
+    auto scatter_kernel =
+        items == 16 ? bucket_scatter_kernel<16> : (items == 8 ? bucket_scatter_kernel<8> : bucket_scatter_kernel<4>);
+    hist_kernel<<<dim3(n_tiles), dim3(kHistThreads), 0, st>>>(unq_inv, n, U, low_bits, high_bins, hist, tile_flags,
+                                                              n_tiles);
     // one entry more than the histogram: it receives the total, the end of the last bucket
     if (exclusive_scan(hist, used, hist, used + 1, scan_ws, st) != hipSuccess) return TXS_ERR_LAUNCH;
     const size_t lds_scatter = (size_t)(kHistWaves + 1) * high_bins * sizeof(int);
     if (low_bits == 0) {
         // a bucket is a voxel: the scatter already gives the final order
-        bucket_scatter_kernel<<<dim3(n_tiles), dim3(kHistThreads), lds_scatter, st>>>(
+        scatter_kernel<<<dim3(n_tiles), dim3(kHistThreads), lds_scatter, st>>>(
             unq_inv, n, U, low_bits, high_bits, hist, tile_flags, n_tiles, n + 1, bucket_start, stats, seg, perm,
             nullptr);
         int rc = txs_plan_presum(seg, n, U, preSum, stream);
@@ -943,8 +1011,8 @@ int txs_plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, i
     }
     // a bucket so full that its workgroups would run long after all others have finished
     // (only a few voxels holding most of the rows do that) sends the call to the general sequence
-    const long giant = (long)kBktMaxSlices * kBktSlice * 2;
-    bucket_scatter_kernel<<<dim3(n_tiles), dim3(kHistThreads), lds_scatter, st>>>(
+    const long giant = kBktGiant;
+    scatter_kernel<<<dim3(n_tiles), dim3(kHistThreads), lds_scatter, st>>>(
         unq_inv, n, U, low_bits, high_bits, hist, tile_flags, n_tiles, giant, bucket_start, stats, nullptr,
         nullptr, reinterpret_cast<int2 *>(pairs1));
     const int low_bins = 1 << low_bits;

@@ -166,7 +166,8 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
 
     // Start value of a running max: -inf, or in reference-tie mode the
     // reference's own -FLT_MAX (scatter_kernel.cu:139), which -inf never beats.
-    const float acc0 = kRef ? TR::to_f(TR::lowest()) : (kMax ? -__builtin_inff() : 0.0f);
+    using AccT = typename std::conditional<kMax, typename TR::max_t, float>::type;
+    const AccT acc0 = kRef ? (AccT)TR::to_m(TR::lowest()) : (AccT)(kMax ? -__builtin_inff() : 0.0f);
     // offset of position l inside its voxel, for the reference's tie key; an
     // ordinary run always starts inside the range, a heavy one may not
     auto rel_of_run_start = [&](int sg, int l) -> int {
@@ -174,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
         const int u = sg & kIdMask;
         return ((unsigned)u < (unsigned)U) ? (t0 - 1 + l) - preSum[u] : 0;
     };
-    float acc[VEC];
+    AccT acc[VEC];
     int idx[VEC];
     int cur = seg_s[la];
     int run_l0 = la;
@@ -220,7 +221,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                 Pack<int, VEC> ai;
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) {
-                    r.v[k] = idx[k] >= 0 ? TR::from_f(acc[k]) : TR::lowest();
+                    r.v[k] = idx[k] >= 0 ? TR::from_m(acc[k]) : TR::lowest();
                     ai.v[k] = idx[k];
                     if (kRef && idx[k] >= 0) ai.v[k] = row_at(run_l0 + ref_rel(idx[k], ref_log2) - rel0);
                 }
@@ -235,7 +236,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 if constexpr (kMax) {
-                    sv[k] = idx[k] >= 0 ? (((unsigned long long)ordered_bits(acc[k]) << 32) |
+                    sv[k] = idx[k] >= 0 ? (((unsigned long long)ordered_bits((float)acc[k]) << 32) |
                                            (unsigned long long)(0xffffffffu - (unsigned)idx[k]))
                                         : 0ull;
                 } else {
@@ -267,8 +268,8 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
         const int tag = kRef ? ref_key(rel0 + (l - run_l0), ref_log2) : row;
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
-            const float x = TR::to_f(v.v[k]);
-            if (kMax) {
+            if constexpr (kMax) {
+                const AccT x = TR::to_m(v.v[k]);
                 // strict '>': the first row wins ties, NaN never wins.  Reference-tie
                 // mode also takes an equal value whose key is smaller.
                 bool take = x > acc[k];
@@ -277,6 +278,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                 acc[k] = take ? x : acc[k];
                 idx[k] = take ? tag : idx[k];
             } else {
+                const float x = TR::to_f(v.v[k]);
                 acc[k] += (!kGate || valid) ? x : 0.0f;
             }
         }

@@ -24,8 +24,14 @@ constexpr int kTableLdsBudget = 144 * 1024;  // bytes of LDS a table may take (1
 #ifndef TXS_TABLE_MAX_WGS
 #define TXS_TABLE_MAX_WGS 1024
 #endif
+#ifndef TXS_TABLE_NT_LOADS
+#define TXS_TABLE_NT_LOADS 1
+#endif
+#ifndef TXS_TABLE_NT_STORES
+#define TXS_TABLE_NT_STORES 0
+#endif
 #ifndef TXS_TABLE_UNROLL
-#define TXS_TABLE_UNROLL 4
+#define TXS_TABLE_UNROLL 2
 #endif
 constexpr int kTableUnroll = TXS_TABLE_UNROLL;  // rows per lane in flight
 constexpr int kReduceThreads = 1024;
@@ -62,23 +68,30 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
     const long r0 = (long)blockIdx.x * rows_per_wg;
     const int r_end = (int)min((long)N, r0 + rows_per_wg);
     if (col < C) {
-        for (int rb = (int)r0 + g; rb < r_end; rb += G * kTableUnroll) {
+        // Two batches of kTableUnroll rows per lane: the next one is on its way from memory
+        // while the current one goes into the table.
+        struct Batch {
             int u[kTableUnroll];
             Pack<raw, VEC> v[kTableUnroll];
+        };
+        const int step = G * kTableUnroll;
+        auto issue = [&](Batch &b, int rb) {
 #pragma unroll
             for (int k = 0; k < kTableUnroll; ++k) {
                 const int r = min(rb + k * G, r_end - 1);  // slots past the span re-load its last row
-                u[k] = inv[r] & kIdMask;
-                v[k] = ld_stream<raw, VEC>(feats + (size_t)r * C + col);
+                b.u[k] = inv[r] & kIdMask;
+                b.v[k] = TXS_TABLE_NT_LOADS ? ld_stream<raw, VEC>(feats + (size_t)r * C + col) : ld<raw, VEC>(feats + (size_t)r * C + col);
             }
+        };
+        auto consume = [&](const Batch &b, int rb) {
 #pragma unroll
             for (int k = 0; k < kTableUnroll; ++k) {
                 const int r = rb + k * G;
-                if (r >= r_end || (unsigned)u[k] >= (unsigned)U) continue;
-                const int cell = u[k] * stride + col;
+                if (r >= r_end || (unsigned)b.u[k] >= (unsigned)U) continue;
+                const int cell = b.u[k] * stride + col;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    const float x = TR::to_f(v[k].v[e]);
+                    const float x = TR::to_f(b.v[k].v[e]);
                     if constexpr (kMax) {
                         if (x == x)  // NaN never wins
                             __hip_atomic_fetch_max(tkey + cell + e,
@@ -90,6 +103,27 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
                                                __HIP_MEMORY_SCOPE_WORKGROUP);
                     }
                 }
+            }
+        };
+        int rb = (int)r0 + g;
+        if (rb < r_end) {
+            Batch b0, b1;
+            issue(b0, rb);
+            for (;;) {
+                if (rb + step >= r_end) {
+                    consume(b0, rb);
+                    break;
+                }
+                issue(b1, rb + step);
+                consume(b0, rb);
+                rb += step;
+                if (rb + step >= r_end) {
+                    consume(b1, rb);
+                    break;
+                }
+                issue(b0, rb + step);
+                consume(b1, rb);
+                rb += step;
             }
         }
     }
@@ -122,8 +156,10 @@ __global__ __launch_bounds__(kReduceThreads) void table_reduce_kernel(
     constexpr bool kMax = OP == TXS_MAX;
     using Cell = typename std::conditional<kMax, unsigned long long, float>::type;  // as the forward stored it
     using Acc = typename std::conditional<kMax, unsigned long long, double>::type;
-    constexpr int kCellsPerWg = kReduceThreads / kReduceSplit;
-    __shared__ Acc part_s[kReduceSplit][kCellsPerWg];
+    // a wave reads whole 128-byte lines of a partial: 16 packed cells or 32 floats
+    constexpr int kSplit = kMax ? kReduceSplit : kReduceSplit / 2;
+    constexpr int kCellsPerWg = kReduceThreads / kSplit;
+    __shared__ Acc part_s[kSplit][kCellsPerWg];
     const int cl = (int)threadIdx.x % kCellsPerWg, wl = (int)threadIdx.x / kCellsPerWg;
     const long cell = (long)blockIdx.x * kCellsPerWg + cl;
     const long total = (long)U * C;
@@ -131,11 +167,11 @@ __global__ __launch_bounds__(kReduceThreads) void table_reduce_kernel(
     Acc acc = Acc(0);
     if (cell < total) {
         // kReduceLoads independent loads in flight per lane
-        for (int w0 = wl; w0 < num_parts; w0 += kReduceSplit * kReduceLoads) {
+        for (int w0 = wl; w0 < num_parts; w0 += kSplit * kReduceLoads) {
             Cell x[kReduceLoads];
 #pragma unroll
             for (int k = 0; k < kReduceLoads; ++k) {
-                const int w = w0 + k * kReduceSplit;
+                const int w = w0 + k * kSplit;
                 x[k] = w < num_parts ? p[(size_t)w * total + cell] : Cell(0);
             }
 #pragma unroll
@@ -146,12 +182,13 @@ __global__ __launch_bounds__(kReduceThreads) void table_reduce_kernel(
     }
     part_s[wl][cl] = acc;
     __syncthreads();
-    // second level in a fixed order: lanes 0..7 of a cell each fold 8 of the 64 values, lane 0 folds those
+    // second level in a fixed order: lanes 0..7 of a cell each fold an eighth of the values, lane 0 folds those
+    constexpr int kFold = kSplit / 8;
     if (wl < 8) {
-        acc = part_s[wl * 8][cl];
+        acc = part_s[wl * kFold][cl];
 #pragma unroll
-        for (int k = 1; k < 8; ++k) {
-            const Acc x = part_s[wl * 8 + k][cl];
+        for (int k = 1; k < kFold; ++k) {
+            const Acc x = part_s[wl * kFold + k][cl];
             if constexpr (kMax) acc = x > acc ? x : acc; else acc += x;
         }
     }
@@ -197,13 +234,28 @@ __global__ __launch_bounds__(kTableThreads) void table_bwd_kernel(
     int *at = reinterpret_cast<int *>(reinterpret_cast<char *>(table_lds) +
                                       (((size_t)U * stride * sizeof(raw) + 31) & ~(size_t)31));
     const int total = U * C;
-    for (int i = threadIdx.x; i < total; i += kTableThreads) {
-        const int uu = i / C, c = i - uu * C;
-        raw x = g[i];
-        if (OP == TXS_MEAN)  // one division per output cell, as (g / unq_cnts) in the reference
-            x = TR::from_f(TR::to_f(x) / (float)(preSum[uu + 1] - preSum[uu]));
-        gt[uu * stride + c] = x;
-        if (OP == TXS_MAX) at[uu * stride + c] = arg[i];
+    constexpr int kStage = 4;  // independent loads per lane while the tables are staged
+    for (int i0 = threadIdx.x; i0 < total; i0 += kTableThreads * kStage) {
+        raw x[kStage];
+        int a[kStage], cnt[kStage], uu[kStage];
+#pragma unroll
+        for (int k = 0; k < kStage; ++k) {
+            const int i = min(i0 + k * kTableThreads, total - 1);
+            uu[k] = i / C;
+            x[k] = g[i];
+            if (OP == TXS_MEAN) cnt[k] = preSum[uu[k] + 1] - preSum[uu[k]];
+            if (OP == TXS_MAX) a[k] = arg[i];
+        }
+#pragma unroll
+        for (int k = 0; k < kStage; ++k) {
+            const int i = i0 + k * kTableThreads;
+            if (i >= total) break;
+            const int c = i - uu[k] * C;
+            if (OP == TXS_MEAN)  // one division per output cell, as (g / unq_cnts) in the reference
+                x[k] = TR::from_f(TR::to_f(x[k]) / (float)cnt[k]);
+            gt[uu[k] * stride + c] = x[k];
+            if (OP == TXS_MAX) at[uu[k] * stride + c] = a[k];
+        }
     }
     __syncthreads();
 
@@ -214,10 +266,13 @@ __global__ __launch_bounds__(kTableThreads) void table_bwd_kernel(
     if (col >= C) return;
     const long r0 = (long)blockIdx.x * rows_per_wg;
     const int r_end = (int)min((long)N, r0 + rows_per_wg);
-    for (int rb = (int)r0 + grp; rb < r_end; rb += G * kTableUnroll) {
-        int u[kTableUnroll];
+    // the voxel ids of the next batch of rows are fetched while the current batch is written
+    const int step = G * kTableUnroll;
+    auto issue = [&](int (&u)[kTableUnroll], int rb) {
 #pragma unroll
         for (int k = 0; k < kTableUnroll; ++k) u[k] = inv[min(rb + k * G, r_end - 1)] & kIdMask;
+    };
+    auto emit = [&](const int (&u)[kTableUnroll], int rb) {
 #pragma unroll
         for (int k = 0; k < kTableUnroll; ++k) {
             const int r = rb + k * G;
@@ -234,8 +289,28 @@ __global__ __launch_bounds__(kTableThreads) void table_bwd_kernel(
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) o.v[e] = TR::zero();
             }
-            st_stream<raw, VEC>(gin + (size_t)r * C + col, o);
+            if (TXS_TABLE_NT_STORES) st_stream<raw, VEC>(gin + (size_t)r * C + col, o); else st<raw, VEC>(gin + (size_t)r * C + col, o);
         }
+    };
+    int rb = (int)r0 + grp;
+    if (rb >= r_end) return;
+    int u0[kTableUnroll], u1[kTableUnroll];
+    issue(u0, rb);
+    for (;;) {
+        if (rb + step >= r_end) {
+            emit(u0, rb);
+            break;
+        }
+        issue(u1, rb + step);
+        emit(u0, rb);
+        rb += step;
+        if (rb + step >= r_end) {
+            emit(u1, rb);
+            break;
+        }
+        issue(u0, rb + step);
+        emit(u1, rb);
+        rb += step;
     }
 }
 
@@ -278,7 +353,7 @@ hipError_t launch_table_fwd(const txs_detail::TablePlan &tp, hipStream_t st, con
     kernel<<<dim3(tp.workgroups), dim3(kTableThreads), tp.lds_bytes, st>>>(
         (const raw *)feats, inv, partials, N, C, U, tp.lpr_log2, tp.stride, tp.rows_per_wg);
     const long total = (long)U * C;
-    constexpr int kCellsPerWg = kReduceThreads / kReduceSplit;
+    constexpr int kCellsPerWg = kReduceThreads / (OP == TXS_MAX ? kReduceSplit : kReduceSplit / 2);
     table_reduce_kernel<TR, OP><<<dim3((unsigned)((total + kCellsPerWg - 1) / kCellsPerWg)), dim3(kReduceThreads), 0, st>>>(
         (const raw *)feats, partials, preSum, (raw *)out, arg, tp.workgroups, N, C, U);
     return hipGetLastError();

@@ -37,6 +37,9 @@ namespace {
 #ifndef TXS_HALF_VEC_BYTES
 #define TXS_HALF_VEC_BYTES 8
 #endif
+#ifndef TXS_F16_NATIVE_MAX
+#define TXS_F16_NATIVE_MAX 1
+#endif
 #ifndef TXS_NT_LOADS
 #define TXS_NT_LOADS 1
 #endif
@@ -66,6 +69,10 @@ struct F32 {
     static __device__ __forceinline__ raw from_f(float x) { return x; }
     static __device__ __forceinline__ raw lowest() { return -3.402823466e+38f; }
     static __device__ __forceinline__ raw zero() { return 0.0f; }
+    // type a running max is kept and compared in (exact for every value of raw)
+    using max_t = float;
+    static __device__ __forceinline__ max_t to_m(raw x) { return x; }
+    static __device__ __forceinline__ raw from_m(max_t x) { return x; }
 };
 struct F16 {
     using raw = _Float16;
@@ -73,6 +80,15 @@ struct F16 {
     static __device__ __forceinline__ raw from_f(float x) { return (_Float16)x; }  // RNE
     static __device__ __forceinline__ raw lowest() { return (_Float16)(-65504.0f); }
     static __device__ __forceinline__ raw zero() { return (_Float16)0.0f; }
+#if TXS_F16_NATIVE_MAX
+    using max_t = _Float16;  // compared with the 16-bit compare instructions, no widening
+    static __device__ __forceinline__ max_t to_m(raw x) { return x; }
+    static __device__ __forceinline__ raw from_m(max_t x) { return x; }
+#else
+    using max_t = float;
+    static __device__ __forceinline__ max_t to_m(raw x) { return (float)x; }
+    static __device__ __forceinline__ raw from_m(max_t x) { return (_Float16)x; }
+#endif
 };
 struct BF16 {
     using raw = unsigned short;
@@ -85,6 +101,9 @@ struct BF16 {
     }
     static __device__ __forceinline__ raw lowest() { return (raw)0xff7f; }
     static __device__ __forceinline__ raw zero() { return (raw)0; }
+    using max_t = float;
+    static __device__ __forceinline__ max_t to_m(raw x) { return to_f(x); }
+    static __device__ __forceinline__ raw from_m(max_t x) { return from_f(x); }
 };
 
 // VEC consecutive elements moved by one lane with a single memory instruction.
