@@ -87,8 +87,9 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     unsigned long long *__restrict__ scratch, const int *__restrict__ preSum, int N, int C, int U,
     int lpr_log2, int ref_log2) {
     using raw = typename TR::raw;
-    constexpr int kBatch = sizeof(raw) == 2 ? kBatchHalf : ::kBatch;
     constexpr bool kMax = OP == TXS_MAX || OP == TXS_MAX_REFTIE;
+    // (the fp16 running max keeps packed halves and has registers to spare for a deeper batch)
+    constexpr int kBatch = sizeof(raw) == 2 ? ((kMax && std::is_same<TR, F16>::value) ? kBatchHalfMax : kBatchHalf) : ::kBatch;
     constexpr bool kRef = OP == TXS_MAX_REFTIE;  // idx[] then holds ref_key, not a row
     extern __shared__ int lds[];
     const int G = kThreads >> lpr_log2;
@@ -266,6 +267,16 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
             }
         }
         const int tag = kRef ? ref_key(rel0 + (l - run_l0), ref_log2) : row;
+        if constexpr (!kMax && !kGate && TXS_F16_FMA_MIX && std::is_same<TR, F16>::value && VEC % 2 == 0) {
+            unsigned w[VEC / 2 > 0 ? VEC / 2 : 1];
+            __builtin_memcpy(w, &v, sizeof(unsigned) * (VEC / 2));
+#pragma unroll
+            for (int k = 0; k < VEC / 2; ++k) {
+                acc[2 * k] = add_f16_lo(acc[2 * k], w[k]);
+                acc[2 * k + 1] = add_f16_hi(acc[2 * k + 1], w[k]);
+            }
+            return;
+        }
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
             if constexpr (kMax) {

@@ -32,13 +32,19 @@ namespace {
 #define TXS_BATCH_HALF TXS_BATCH
 #endif
 #ifndef TXS_BATCH_BWD_HALF
-#define TXS_BATCH_BWD_HALF TXS_BATCH_BWD
+#define TXS_BATCH_BWD_HALF 8
 #endif
 #ifndef TXS_HALF_VEC_BYTES
 #define TXS_HALF_VEC_BYTES 8
 #endif
 #ifndef TXS_F16_NATIVE_MAX
 #define TXS_F16_NATIVE_MAX 1
+#endif
+#ifndef TXS_F16_FMA_MIX
+#define TXS_F16_FMA_MIX 1
+#endif
+#ifndef TXS_BATCH_HALF_MAX
+#define TXS_BATCH_HALF_MAX 6
 #endif
 #ifndef TXS_NT_LOADS
 #define TXS_NT_LOADS 1
@@ -55,6 +61,7 @@ constexpr int kBatchBwd = TXS_BATCH_BWD;
 constexpr int kBatch = TXS_BATCH;    // rows per load batch of a lane group (two batches in flight)
 constexpr int kBatchHalf = TXS_BATCH_HALF;         // the same for the 2-byte types
 constexpr int kBatchBwdHalf = TXS_BATCH_BWD_HALF;
+constexpr int kBatchHalfMax = TXS_BATCH_HALF_MAX;  // forward max of fp16
 constexpr int kHalfVecBytes = TXS_HALF_VEC_BYTES;  // bytes one lane moves per row for fp16 / bf16
 constexpr int kHeavyDefault = 64;    // voxels above this many rows use the atomic path
 constexpr int kTableMinRowsPerVoxel = 512;  // table mode needs at least this many rows per voxel on average
@@ -105,6 +112,20 @@ struct BF16 {
     static __device__ __forceinline__ max_t to_m(raw x) { return to_f(x); }
     static __device__ __forceinline__ raw from_m(max_t x) { return from_f(x); }
 };
+
+// acc + (float)half taken from the low / high 16 bits of a packed word, in one instruction
+// (the mixed-precision FMA: half operand times 1.0f plus an fp32 accumulator; the product is
+// exact, so the result is the correctly rounded fp32 sum, as a widening followed by an add)
+__device__ __forceinline__ float add_f16_lo(float acc, unsigned packed) {
+    float r;
+    asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "v"(acc));
+    return r;
+}
+__device__ __forceinline__ float add_f16_hi(float acc, unsigned packed) {
+    float r;
+    asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "v"(acc));
+    return r;
+}
 
 // VEC consecutive elements moved by one lane with a single memory instruction.
 template <typename T, int VEC>
