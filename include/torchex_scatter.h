@@ -249,6 +249,17 @@ int txs_dynamic_point_pool(const float *rois, const float *pts, int64_t num_boxe
                            float *out_pts_feats, int32_t *num_out, void *stream);
 int64_t txs_dpp_workspace_len(int64_t num_pts, int64_t num_boxes);
 
+/* The same for a batch of samples held in one pair of tensors.  Replaces
+ * dynamic_point_pool_mixed_launcher (torchex/src/dynamic_point_pool/dynamic_point_pool.cpp:108-164,
+ * kernel generate_pts_mask_for_box3d_mixed, dynamic_point_pool_kernel.cu:173-212): rois_batch
+ * [num_boxes] and pts_batch [num_pts] give the sample of every box and point, and a point is
+ * tested only against the boxes of its own sample.  Both NULL: txs_dynamic_point_pool. */
+int txs_dynamic_point_pool_mixed(const float *rois, const int32_t *rois_batch, const float *pts,
+                                 const int32_t *pts_batch, int64_t num_boxes, int64_t num_pts,
+                                 const float *extra_wlh, int32_t max_pts_per_box, int64_t max_all_pts,
+                                 int32_t *workspace, int64_t *out_pts_idx, int64_t *out_roi_idx,
+                                 float *out_pts_feats, int32_t *num_out, void *stream);
+
 /* Hash table of int32 (key, value) pairs.  Replace build_hash_table_launcher /
  * probe_hash_table_launcher (torchex/src/grid_hash/grid_hash.cpp:14-27, kernels
  * grid_hash_kernel.cu:19-49, probing of src/utils/functions.cuh:30-64).

@@ -213,16 +213,20 @@ def voxelize(points, voxel_size, range_lo, dims):
     return coors, keys
 
 
-def dynamic_point_pool(rois, pts, extra_wlh, max_pts, max_all):
+def dynamic_point_pool(rois, pts, extra_wlh, max_pts, max_all, rois_batch=None, pts_batch=None):
     r = _f32(rois)
     p = _f32(pts)
     e = _f32(extra_wlh)
     idx = np.full(max_all, -1, dtype=np.int64)
     roi = np.full(max_all, -1, dtype=np.int64)
     feats = np.zeros((max_all, 13), dtype=np.float32)
-    lib().orc_dynamic_point_pool.restype = ctypes.c_int64
-    m = lib().orc_dynamic_point_pool(_p(r), _ll(r.shape[0]), _p(p), _ll(p.shape[0]), _p(e),
-                                     ctypes.c_int(int(max_pts)), _ll(max_all), _p(idx), _p(roi), _p(feats))
+    rb = _i32(rois_batch) if rois_batch is not None else None
+    pb = _i32(pts_batch) if pts_batch is not None else None
+    assert (rb is None) == (pb is None)
+    lib().orc_dynamic_point_pool_mixed.restype = ctypes.c_int64
+    m = lib().orc_dynamic_point_pool_mixed(_p(r), _p(rb) if rb is not None else None, _ll(r.shape[0]), _p(p),
+                                           _p(pb) if pb is not None else None, _ll(p.shape[0]), _p(e),
+                                           ctypes.c_int(int(max_pts)), _ll(max_all), _p(idx), _p(roi), _p(feats))
     return idx[:m], roi[:m], feats[:m]
 
 

@@ -394,10 +394,14 @@ void orc_voxelize(const float *points, int64_t n, int64_t stride, const float *l
  * wrapper comment calls the usual one.  Mixed float/double arithmetic as
  * written there; the rotation terms cos/sin(rz + pi/2) are evaluated in double
  * and rounded to float (the device's cosf/sinf is within an ulp of that).
+ * rois_batch / pts_batch (both NULL, or both given): the sample every box and point
+ * belongs to; a pair is tested only when they agree, as in
+ * generate_pts_mask_for_box3d_mixed (dynamic_point_pool_kernel.cu:173-212).
  * Returns the number of entries written. */
-int64_t orc_dynamic_point_pool(const float *rois, int64_t B, const float *pts, int64_t P,
-                               const float *extra_wlh, int max_pts, int64_t max_all,
-                               int64_t *out_pts_idx, int64_t *out_roi_idx, float *out_feats) {
+int64_t orc_dynamic_point_pool_mixed(const float *rois, const int32_t *rois_batch, int64_t B,
+                                     const float *pts, const int32_t *pts_batch, int64_t P,
+                                     const float *extra_wlh, int max_pts, int64_t max_all,
+                                     int64_t *out_pts_idx, int64_t *out_roi_idx, float *out_feats) {
     int64_t global = 0;
     for (int64_t b = 0; b < B; ++b) {
         const float *r = rois + b * 7;
@@ -408,6 +412,7 @@ int64_t orc_dynamic_point_pool(const float *rois, int64_t B, const float *pts, i
         const float cosa = (float)cos((double)rot), sina = (float)sin((double)rot);
         int in_box_counter = 0;
         for (int64_t p = 0; p < P; ++p) {
+            if (rois_batch && pts_batch[p] != rois_batch[b]) continue;
             const float x = pts[p * 3], y = pts[p * 3 + 1], z = pts[p * 3 + 2];
             if ((double)fabsf(z - cz) > (double)large_h / 2.0) continue;
             volatile float sx = x - cx, sy = y - cy;
@@ -440,6 +445,12 @@ int64_t orc_dynamic_point_pool(const float *rois, int64_t B, const float *pts, i
         }
     }
     return global < max_all ? global : max_all;
+}
+int64_t orc_dynamic_point_pool(const float *rois, int64_t B, const float *pts, int64_t P,
+                               const float *extra_wlh, int max_pts, int64_t max_all,
+                               int64_t *out_pts_idx, int64_t *out_roi_idx, float *out_feats) {
+    return orc_dynamic_point_pool_mixed(rois, NULL, B, pts, NULL, P, extra_wlh, max_pts, max_all, out_pts_idx,
+                                        out_roi_idx, out_feats);
 }
 
 /* ---- grid hash ------------------------------------------------------------

@@ -191,6 +191,33 @@ def test_dynamic_point_pool(B, P, cap, max_all, extra):
     assert idx.shape[0] <= max_all and torch.bincount(roi).max().item() <= cap
 
 
+@pytest.mark.parametrize("cap,max_all", [(10 ** 6, 10 ** 6), (5, 300)])
+def test_dynamic_point_pool_mixed_batches(cap, max_all):
+    """Boxes and points of several samples in one call (the reference extension's
+    dynamic_point_pool_mixed_gpu): bit-exact against the oracle, never a pair across
+    samples, and with every index in one sample the same as the plain op."""
+    T = tx()
+    rois, pts = _boxes_and_points(123, 60, 50_000)
+    g = torch.Generator().manual_seed(9)
+    rb = torch.randint(0, 4, (60,), generator=g)
+    pb = torch.randint(0, 4, (50_000,), generator=g)
+    extra = [0.4, 0.4, 0.2]
+    say(f"[case] dynamic_point_pool mixed cap={cap} max_all={max_all}")
+    idx, roi, feats = T.dynamic_point_pool(rois.to(DEV), pts.to(DEV), extra, cap, max_all,
+                                           rois_batch=rb.to(DEV), pts_batch=pb.to(DEV))
+    wi, wr, wf = orc.dynamic_point_pool(rois.numpy(), pts.numpy(), extra, cap, max_all, rb.numpy(), pb.numpy())
+    assert wi.shape[0] > 50
+    assert np.array_equal(idx.cpu().numpy(), wi) and np.array_equal(roi.cpu().numpy(), wr)
+    assert np.array_equal(feats.cpu().numpy().view(np.uint32), wf.view(np.uint32))
+    assert torch.equal(rb[roi.cpu()], pb[idx.cpu()])
+    zr, zp = torch.zeros_like(rb).to(DEV), torch.zeros_like(pb).to(DEV)
+    a = T.dynamic_point_pool(rois.to(DEV), pts.to(DEV), extra, cap, max_all, rois_batch=zr, pts_batch=zp)
+    b = T.dynamic_point_pool(rois.to(DEV), pts.to(DEV), extra, cap, max_all)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    with pytest.raises(AssertionError):
+        T.dynamic_point_pool(rois.to(DEV), pts.to(DEV), extra, cap, max_all, rois_batch=zr)
+
+
 def test_dynamic_point_pool_corner_points():
     """Points placed a hair inside and outside the corners and edge midpoints of the
     rotated (enlarged) boxes: the farthest places from a box centre that still count,

@@ -449,6 +449,36 @@ def test_dynamic_point_pool_oracle_geometry():
     assert np.array_equal(i2, idx[keep]) and np.array_equal(f2, feats[keep])
 
 
+def test_dynamic_point_pool_oracle_mixed_batches():
+    """A batch held in one pair of tensors (generate_pts_mask_for_box3d_mixed,
+    dynamic_point_pool_kernel.cu:173-212) gives what the single-sample op gives sample by
+    sample: the pairs of sample s are the op's output on that sample's boxes and points, with
+    the indices mapped back; a pair of different samples never appears."""
+    rois, pts = _boxes_and_points(5)
+    g = torch.Generator().manual_seed(6)
+    rb = torch.randint(0, 3, (rois.shape[0],), generator=g).numpy().astype(np.int32)
+    pb = torch.randint(0, 3, (pts.shape[0],), generator=g).numpy().astype(np.int32)
+    extra = [0.5, 0.5, 0.3]
+    idx, roi, feats = orc.dynamic_point_pool(rois.numpy(), pts.numpy(), extra, 10 ** 6, 10 ** 6, rb, pb)
+    assert idx.shape[0] > 100 and np.array_equal(rb[roi], pb[idx])
+    parts = []
+    for s_ in range(3):
+        bsel, psel = np.nonzero(rb == s_)[0], np.nonzero(pb == s_)[0]
+        i1, r1, f1 = orc.dynamic_point_pool(rois.numpy()[bsel], pts.numpy()[psel], extra, 10 ** 6, 10 ** 6)
+        parts.append((psel[i1], bsel[r1], f1))
+    wi = np.concatenate([p[0] for p in parts])
+    wr = np.concatenate([p[1] for p in parts])
+    wf = np.concatenate([p[2] for p in parts])
+    order = np.lexsort((wi, wr))               # the mixed op emits in (box, point) order
+    assert np.array_equal(idx, wi[order]) and np.array_equal(roi, wr[order])
+    assert np.array_equal(feats.view(np.uint32), wf[order].view(np.uint32))
+    # all in one sample: the plain op
+    z_r, z_p = np.zeros_like(rb), np.zeros_like(pb)
+    a = orc.dynamic_point_pool(rois.numpy(), pts.numpy(), extra, 9, 400, z_r, z_p)
+    b = orc.dynamic_point_pool(rois.numpy(), pts.numpy(), extra, 9, 400)
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))
+
+
 def test_grid_hash_oracle():
     rng = np.random.default_rng(5)
     keys = rng.choice(10 ** 7, size=3000, replace=False).astype(np.int32)

@@ -181,24 +181,30 @@ __device__ __forceinline__ int dpp_test(const DppBox &bx, float x, float y, floa
 constexpr int kDppBoxesPerWg = 8;
 
 // hits per (box, tile); grid (tiles, groups of boxes)
+// (pts_batch / rois_batch, both NULL or both given: a point meets only the boxes of its own
+// sample, generate_pts_mask_for_box3d_mixed, dynamic_point_pool_kernel.cu:173-212)
 __global__ __launch_bounds__(kThreads) void dpp_count_kernel(const float *__restrict__ pts, int P,
                                                              const DppBox *__restrict__ boxes, int B,
-                                                             int n_tiles, int *__restrict__ counts) {
+                                                             int n_tiles, int *__restrict__ counts,
+                                                             const int *__restrict__ pts_batch,
+                                                             const int *__restrict__ rois_batch) {
     __shared__ int cnt[kDppBoxesPerWg];
     const int p = blockIdx.x * kThreads + threadIdx.x;
     const int b0 = blockIdx.y * kDppBoxesPerWg;
     if (threadIdx.x < kDppBoxesPerWg) cnt[threadIdx.x] = 0;
     __syncthreads();
     float x = 0.f, y = 0.f, z = 0.f;
+    int sample = 0;
     if (p < P) {
         x = pts[(size_t)p * 3];
         y = pts[(size_t)p * 3 + 1];
         z = pts[(size_t)p * 3 + 2];
+        if (pts_batch) sample = pts_batch[p];
     }
     for (int bb = 0; bb < kDppBoxesPerWg && b0 + bb < B; ++bb) {
         const DppBox bx = boxes[b0 + bb];
         bool hit = false;
-        if (p < P && dpp_near(bx, x, y)) {
+        if (p < P && (!rois_batch || rois_batch[b0 + bb] == sample) && dpp_near(bx, x, y)) {
             float lx, ly;
             hit = dpp_test(bx, x, y, z, lx, ly) > 0;
         }
@@ -233,17 +239,19 @@ __global__ __launch_bounds__(kThreads) void dpp_write_kernel(
     const float *__restrict__ pts, int P, const DppBox *__restrict__ boxes, int B, int n_tiles,
     const int *__restrict__ scanned, const int *__restrict__ box_base, int cap, int max_all,
     long long *__restrict__ out_pts_idx, long long *__restrict__ out_roi_idx,
-    float *__restrict__ out_feats) {
+    float *__restrict__ out_feats, const int *__restrict__ pts_batch, const int *__restrict__ rois_batch) {
 #pragma clang fp contract(off)
     __shared__ int wsum[kDppBoxesPerWg][kThreads / 64];
     const int b0 = blockIdx.y * kDppBoxesPerWg;
     const int p = blockIdx.x * kThreads + threadIdx.x;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     float x = 0.f, y = 0.f, z = 0.f;
+    int sample = 0;
     if (p < P) {
         x = pts[(size_t)p * 3];
         y = pts[(size_t)p * 3 + 1];
         z = pts[(size_t)p * 3 + 2];
+        if (pts_batch) sample = pts_batch[p];
     }
     // phase 1: the test against every box of the group (2 result bits per box) and the
     // hits of each wave
@@ -251,7 +259,7 @@ __global__ __launch_bounds__(kThreads) void dpp_write_kernel(
     for (int bb = 0; bb < kDppBoxesPerWg && b0 + bb < B; ++bb) {
         const DppBox bx = boxes[b0 + bb];
         int flag = 0;
-        if (p < P && dpp_near(bx, x, y)) {
+        if (p < P && (!rois_batch || rois_batch[b0 + bb] == sample) && dpp_near(bx, x, y)) {
             float lx, ly;
             flag = dpp_test(bx, x, y, z, lx, ly);
         }
@@ -414,6 +422,16 @@ int txs_dynamic_point_pool(const float *rois, const float *pts, int64_t num_boxe
                            const float *extra_wlh, int32_t max_pts_per_box, int64_t max_all_pts,
                            int32_t *workspace, int64_t *out_pts_idx, int64_t *out_roi_idx,
                            float *out_pts_feats, int32_t *num_out, void *stream) {
+    return txs_dynamic_point_pool_mixed(rois, nullptr, pts, nullptr, num_boxes, num_pts, extra_wlh,
+                                        max_pts_per_box, max_all_pts, workspace, out_pts_idx, out_roi_idx,
+                                        out_pts_feats, num_out, stream);
+}
+
+int txs_dynamic_point_pool_mixed(const float *rois, const int32_t *rois_batch, const float *pts,
+                                 const int32_t *pts_batch, int64_t num_boxes, int64_t num_pts,
+                                 const float *extra_wlh, int32_t max_pts_per_box, int64_t max_all_pts,
+                                 int32_t *workspace, int64_t *out_pts_idx, int64_t *out_roi_idx,
+                                 float *out_pts_feats, int32_t *num_out, void *stream) {
     if (!fits_i32(num_boxes) || !fits_i32(num_pts) || !fits_i32(max_all_pts) || max_pts_per_box < 0 ||
         !extra_wlh || !num_out)
         return TXS_ERR_INVALID_ARG;
@@ -422,7 +440,8 @@ int txs_dynamic_point_pool(const float *rois, const float *pts, int64_t num_boxe
         fill_i32_kernel<<<dim3(1), dim3(64), 0, st>>>(num_out, 1, 0);
         return status_of(hipGetLastError());
     }
-    if (!rois || !pts || !workspace || !out_pts_idx || !out_roi_idx || !out_pts_feats)
+    if (!rois || !pts || !workspace || !out_pts_idx || !out_roi_idx || !out_pts_feats ||
+        ((rois_batch == nullptr) != (pts_batch == nullptr)))
         return TXS_ERR_INVALID_ARG;
     const int B = (int)num_boxes, P = (int)num_pts;
     const int n_tiles = (P + kThreads - 1) / kThreads;
@@ -435,13 +454,14 @@ int txs_dynamic_point_pool(const float *rois, const float *pts, int64_t num_boxe
     dpp_box_kernel<<<dim3(blocks_for(B)), dim3(kThreads), 0, st>>>(rois, B, extra_wlh[0], extra_wlh[1],
                                                                  extra_wlh[2], boxes);
     const int box_groups = (B + kDppBoxesPerWg - 1) / kDppBoxesPerWg;
-    dpp_count_kernel<<<dim3(n_tiles, box_groups), dim3(kThreads), 0, st>>>(pts, P, boxes, B, n_tiles, counts);
+    dpp_count_kernel<<<dim3(n_tiles, box_groups), dim3(kThreads), 0, st>>>(pts, P, boxes, B, n_tiles, counts,
+                                                                           pts_batch, rois_batch);
     if (exclusive_scan(counts, cells, counts, cells + 1, scan_ws, st) != hipSuccess) return TXS_ERR_LAUNCH;
     dpp_box_base_kernel<<<dim3(1), dim3(kThreads), 0, st>>>(counts, B, n_tiles, max_pts_per_box,
                                                            (int)max_all_pts, box_base, num_out);
     dpp_write_kernel<<<dim3(n_tiles, box_groups), dim3(kThreads), 0, st>>>(
         pts, P, boxes, B, n_tiles, counts, box_base, max_pts_per_box, (int)max_all_pts,
-        (long long *)out_pts_idx, (long long *)out_roi_idx, out_pts_feats);
+        (long long *)out_pts_idx, (long long *)out_roi_idx, out_pts_feats, pts_batch, rois_batch);
     return status_of(hipGetLastError());
 }
 

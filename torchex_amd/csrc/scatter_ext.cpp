@@ -261,11 +261,20 @@ Tensor ingroup_inds(const Tensor &seg, const OptTensor &perm, const Tensor &preS
 
 // dynamic_point_pool(rois [B,7], pts [P,3], extra_wlh, max_pts_per_box, max_all_pts)
 // -> (out_pts_idx int64 [M], out_roi_idx int64 [M], out_pts_feats float [M,13]); one host sync to read M.
+// rois_batch [B] / pts_batch [P] (int32, both or neither): the sample of every box and point.
 std::tuple<Tensor, Tensor, Tensor> dynamic_point_pool(const Tensor &rois, const Tensor &pts,
                                                       std::vector<double> extra_wlh,
-                                                      int64_t max_pts_per_box, int64_t max_all_pts) {
+                                                      int64_t max_pts_per_box, int64_t max_all_pts,
+                                                      const OptTensor &rois_batch, const OptTensor &pts_batch) {
     check_dev(rois, "rois");
     check_dev(pts, "pts");
+    TORCH_CHECK(rois_batch.has_value() == pts_batch.has_value(), "rois_batch and pts_batch go together");
+    if (rois_batch.has_value()) {
+        check_i32(*rois_batch, "rois_batch");
+        check_i32(*pts_batch, "pts_batch");
+        TORCH_CHECK(rois_batch->dim() == 1 && rois_batch->numel() == rois.size(0), "rois_batch must be [num_boxes]");
+        TORCH_CHECK(pts_batch->dim() == 1 && pts_batch->numel() == pts.size(0), "pts_batch must be [num_pts]");
+    }
     TORCH_CHECK(rois.dim() == 2 && rois.size(1) == 7 && rois.scalar_type() == at::kFloat,
                 "rois must be float32 [num_boxes, 7]");
     TORCH_CHECK(pts.dim() == 2 && pts.size(1) == 3 && pts.scalar_type() == at::kFloat,
@@ -281,7 +290,8 @@ std::tuple<Tensor, Tensor, Tensor> dynamic_point_pool(const Tensor &rois, const 
     Tensor roi = at::empty({max_all_pts}, pts.options().dtype(at::kLong));
     Tensor feats = at::empty({max_all_pts, 13}, pts.options());
     Tensor num = at::zeros({1}, iopt);
-    check_status(txs_dynamic_point_pool(B ? rois.data_ptr<float>() : nullptr, P ? pts.data_ptr<float>() : nullptr,
+    check_status(txs_dynamic_point_pool_mixed(B ? rois.data_ptr<float>() : nullptr, opt_i32p(rois_batch),
+                                        P ? pts.data_ptr<float>() : nullptr, opt_i32p(pts_batch),
                                         B, P, extra, (int32_t)max_pts_per_box, max_all_pts, i32w(ws),
                                         max_all_pts ? idx.data_ptr<int64_t>() : nullptr,
                                         max_all_pts ? roi.data_ptr<int64_t>() : nullptr,
@@ -591,7 +601,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("voxel_keys", &voxel_keys, "voxel_keys(points, range_lo, voxel_size, dims) -> (coors, keys, stats)");
     m.def("unique_plan", &unique_plan, "unique_plan(keys, key_bound, heavy_threshold, stats|None)");
     m.def("ingroup_inds", &ingroup_inds, "ingroup_inds(seg, perm|None, preSum, num_unq)");
-    m.def("dynamic_point_pool", &dynamic_point_pool, "dynamic_point_pool(rois, pts, extra_wlh, max_pts_per_box, max_all_pts)");
+    m.def("dynamic_point_pool", &dynamic_point_pool,
+          "dynamic_point_pool(rois, pts, extra_wlh, max_pts_per_box, max_all_pts, rois_batch=None, pts_batch=None)",
+          pybind11::arg("rois"), pybind11::arg("pts"), pybind11::arg("extra_wlh"), pybind11::arg("max_pts_per_box"),
+          pybind11::arg("max_all_pts"), pybind11::arg("rois_batch") = pybind11::none(),
+          pybind11::arg("pts_batch") = pybind11::none());
     m.def("grid_hash_build", &grid_hash_build, "build_table(coors, values) -> table");
     m.def("grid_hash_probe", &grid_hash_probe, "probe_table(coors, table) -> values");
     m.def("make_scratch", &make_scratch, "make_scratch(num_total, channel, num_unq, num_heavy, like): zeroed forward scratch");

@@ -9,7 +9,8 @@ import torch
 from ._native import scatter_ext
 
 
-def dynamic_point_pool(rois, pts, extra_wlh, max_inbox_point, max_all_pts=50000):
+def dynamic_point_pool(rois, pts, extra_wlh, max_inbox_point, max_all_pts=50000, rois_batch=None,
+                       pts_batch=None):
     """Points inside the boxes enlarged by ``extra_wlh`` (dynamic_point_pool_op.py:17-57).
 
     Args:
@@ -17,15 +18,23 @@ def dynamic_point_pool(rois, pts, extra_wlh, max_inbox_point, max_all_pts=50000)
             bottom centre, then ``w, l, h, rz``.
         pts (Tensor): float32 ``[npoints, 3]``.
         extra_wlh (sequence of 3 floats), max_inbox_point (int), max_all_pts (int).
+        rois_batch, pts_batch (Tensor, optional, both or neither): integer ``[N]`` /
+            ``[npoints]`` sample index of every box and point; a point is then matched
+            only with the boxes of its own sample (the extension's
+            ``dynamic_point_pool_mixed_gpu``, src/dynamic_point_pool/dynamic_point_pool.cpp:108-164).
     Returns ``(out_pts_idx int64 [M], out_roi_idx int64 [M], out_pts_feats float32 [M, 13])``.
     Entries come in (box, point) order; the reference's atomic counters leave the order
     (and, under a cap, the surviving subset) to thread timing.  With no hit at all the
     reference returns one placeholder entry (-1, -1, zeros); so does this.
     """
     assert len(rois) > 0
+    assert (rois_batch is None) == (pts_batch is None)
+    if rois_batch is not None:
+        rois_batch = rois_batch.int().contiguous()
+        pts_batch = pts_batch.int().contiguous()
     idx, roi, feats = scatter_ext.dynamic_point_pool(
         rois.contiguous(), pts.contiguous(), [float(v) for v in extra_wlh], int(max_inbox_point),
-        int(max_all_pts))
+        int(max_all_pts), rois_batch, pts_batch)
     if idx.numel() == 0:   # the reference fakes a non-empty output (dynamic_point_pool_op.py:41-45)
         idx = pts.new_full((1,), -1, dtype=torch.long)
         roi = pts.new_full((1,), -1, dtype=torch.long)
