@@ -168,7 +168,10 @@ int txs_plan_special(const int32_t *preSum, int64_t num_unq, int32_t heavy_thres
  * slice of all outputs -- beyond that it runs the calls named above.
  * stats [TXS_STATS_LEN] needs no initialisation for up to 2^22 voxels and must be
  * zero-filled by the caller beyond (zero-filling always is fine); perm is left unwritten when
- * stats[UNSORTED] stays 0.  unq_cnts may be NULL.  plan_ws: int32 workspace of
+ * stats[UNSORTED] stays 0.  unq_cnts may be NULL.  slot_of and heavy_ids may both be NULL
+ * for a caller that wants the order and the offsets only (the ranks of ingroup_inds): no
+ * special-voxel table is made then, seg carries plain ids, and of the statistics only
+ * UNSORTED, OUT_OF_RANGE and NEED_GENERAL are set.  plan_ws: int32 workspace of
  * txs_plan_workspace_len(num_total, num_unq) entries, 8-byte aligned.
  * One bucket holding more than 262,144 rows (a few voxels that own most of the rows)
  * makes the bucket kernels step aside: stats[NEED_GENERAL] is then 1, only

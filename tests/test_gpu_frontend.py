@@ -147,6 +147,17 @@ def test_ingroup_inds():
     s = torch.sort(ids).values.int()
     assert T.ingroup_inds(s.to(DEV)).dtype == torch.int32
     assert np.array_equal(T.ingroup_inds(s.to(DEV)).cpu().numpy(), orc.ingroup_inds(s.numpy()).astype(np.int32))
+    # ids at or beyond the number of elements (not the inverse of a unique) take the pass that
+    # reads the largest id first; any shape is ranked as its flattened view
+    sparse = torch.randint(0, 40, (5_000,), generator=g) * 1_000_003 % 2_000_000_000
+    assert int(sparse.max()) >= 5_000
+    assert np.array_equal(T.ingroup_inds(sparse.to(DEV)).cpu().numpy(), orc.ingroup_inds(sparse.numpy()))
+    two_d = torch.randint(0, 7, (40, 25), generator=g)
+    out = T.ingroup_inds(two_d.to(DEV))
+    assert out.shape == two_d.shape
+    assert np.array_equal(out.cpu().numpy().reshape(-1), orc.ingroup_inds(two_d.reshape(-1).numpy()))
+    with pytest.raises(RuntimeError, match="non-negative"):
+        T.ingroup_inds(torch.tensor([3, -1, 2], device=DEV))
 
 
 # ---------------------------------------------------------- dynamic point pool --

@@ -671,7 +671,7 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
     }
     __syncthreads();
     // ---- statistics, special voxels and their slots (first slice only; as plan_special_kernel)
-    if (j == 0) {
+    if (j == 0 && slot_of != nullptr) {
         int vmax = 0;
         bool mismatch = false;
         if (check_counts) {
@@ -936,11 +936,12 @@ int txs_plan_build_general(const int32_t *unq_inv, int64_t num_total, int64_t nu
     const long n = num_total;
     const int U = (int)num_unq;
     if (n > 0 && (!unq_inv || !plan_ws || !perm || !seg)) return TXS_ERR_INVALID_ARG;
-    if (U > 0 && (!slot_of || !heavy_ids)) return TXS_ERR_INVALID_ARG;
+    if (U > 0 && ((slot_of == nullptr) != (heavy_ids == nullptr))) return TXS_ERR_INVALID_ARG;
     // order/range flags, three-kernel radix passes, CSR offsets, special table, flags
     int rc = txs_plan_check(unq_inv, n, U, stats, stream);
     if (rc == TXS_OK && n > 0 && U > 0) rc = txs_plan_sort(unq_inv, n, U, stats, perm, seg, plan_ws, stream);
     if (rc == TXS_OK) rc = txs_plan_presum(seg, U > 0 ? n : 0, U, preSum, stream);
+    if (slot_of == nullptr) return rc;  // order and offsets only
     if (rc == TXS_OK)
         rc = txs_plan_special(preSum, U, heavy_threshold, unq_cnts, slot_of, heavy_ids, stats, nullptr, nullptr,
                               stream);
@@ -957,8 +958,9 @@ int txs_plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, i
     const long n = num_total;
     const int U = (int)num_unq;
     if (n > 0 && (!unq_inv || !plan_ws || !perm || !seg)) return TXS_ERR_INVALID_ARG;
-    if (U > 0 && (!slot_of || !heavy_ids)) return TXS_ERR_INVALID_ARG;
+    if (U > 0 && ((slot_of == nullptr) != (heavy_ids == nullptr))) return TXS_ERR_INVALID_ARG;
     if (((uintptr_t)plan_ws & 7u) != 0) return TXS_ERR_INVALID_ARG;
+    if (slot_of == nullptr) heavy_threshold = 0x7fffffff;  // no special voxels: no flag bit in seg
     const int bits = radix_bits(U > 1 ? U : 1);
     if (n == 0 || U == 0 || bits > kBucketBitsMax)
         return txs_plan_build_general(unq_inv, num_total, num_unq, heavy_threshold, unq_cnts, plan_ws, perm, seg,
@@ -1003,6 +1005,7 @@ int txs_plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, i
             unq_inv, n, U, low_bits, high_bits, hist, tile_flags, n_tiles, n + 1, bucket_start, stats, seg, perm,
             nullptr);
         int rc = txs_plan_presum(seg, n, U, preSum, stream);
+        if (slot_of == nullptr) return rc;
         if (rc == TXS_OK)
             rc = txs_plan_special(preSum, U, heavy_threshold, unq_cnts, slot_of, heavy_ids, stats, nullptr, nullptr,
                                   stream);

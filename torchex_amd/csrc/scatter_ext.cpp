@@ -259,6 +259,54 @@ Tensor ingroup_inds(const Tensor &seg, const OptTensor &perm, const Tensor &preS
     return out;
 }
 
+// group_ranks(ids) -> int64 ranks, one call for the whole of ingroup_inds: index preparation
+// with the number of rows as the bound of the ids (true for the inverse of a unique; the
+// largest id is then never read back), the rank kernel, one host synchronisation.  Ids at
+// or above the number of rows take a second pass with their true bound.
+Tensor group_ranks(const Tensor &ids_in) {
+    check_dev(ids_in, "group_inds");
+    TORCH_CHECK(ids_in.scalar_type() == at::kInt || ids_in.scalar_type() == at::kLong,
+                "group_inds must be int32 or int64");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(ids_in.device());
+    Tensor ids = ids_in.reshape({-1}).contiguous();
+    if (ids.scalar_type() != at::kInt) ids = ids.to(at::kInt);
+    const int64_t N = ids.numel();
+    Tensor out = at::empty({N}, ids.options().dtype(at::kLong));
+    if (N == 0) return out;
+    void *st = cur_stream(ids);
+    auto attempt = [&](int64_t U) -> bool {
+        Tensor stats = at::zeros({TXS_STATS_LEN}, ids.options());
+        Tensor seg = empty_i32(N, ids), perm = empty_i32(N, ids);
+        Tensor preSum = empty_i32(U + 1, ids);
+        Tensor ws = empty_i32(txs_plan_workspace_len(N, U), ids);
+        const int32_t heavy = txs_default_heavy_threshold();
+        // order and offsets only: no special-voxel table
+        check_status(txs_plan_build(i32p(ids), N, U, heavy, nullptr, i32w(ws), i32w(perm), i32w(seg), i32w(preSum),
+                                    nullptr, nullptr, i32w(stats), st),
+                     "plan_build");
+        std::vector<int64_t> hs = read_stats(stats);
+        if (hs[TXS_STAT_OUT_OF_RANGE]) return false;
+        if (hs[TXS_STAT_NEED_GENERAL]) {
+            stats.zero_();
+            check_status(txs_plan_build_general(i32p(ids), N, U, heavy, nullptr, i32w(ws), i32w(perm), i32w(seg),
+                                                i32w(preSum), nullptr, nullptr, i32w(stats), st),
+                         "plan_build_general");
+            hs = read_stats(stats);
+        }
+        // ids already in order leave perm unwritten: position == row
+        check_status(txs_ingroup_inds(i32p(seg), hs[TXS_STAT_UNSORTED] ? i32p(perm) : nullptr, i32p(preSum), N, U,
+                                      out.data_ptr<int64_t>(), st),
+                     "ingroup_inds");
+        return true;
+    };
+    if (!attempt(N)) {
+        const int64_t lo = ids.min().item<int64_t>(), hi = ids.max().item<int64_t>();
+        TORCH_CHECK(lo >= 0, "group_inds must be non-negative");
+        TORCH_CHECK(attempt(hi + 1), "group_inds could not be ranked");
+    }
+    return out;
+}
+
 // dynamic_point_pool(rois [B,7], pts [P,3], extra_wlh, max_pts_per_box, max_all_pts)
 // -> (out_pts_idx int64 [M], out_roi_idx int64 [M], out_pts_feats float [M,13]); one host sync to read M.
 // rois_batch [B] / pts_batch [P] (int32, both or neither): the sample of every box and point.
@@ -601,6 +649,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("voxel_keys", &voxel_keys, "voxel_keys(points, range_lo, voxel_size, dims) -> (coors, keys, stats)");
     m.def("unique_plan", &unique_plan, "unique_plan(keys, key_bound, heavy_threshold, stats|None)");
     m.def("ingroup_inds", &ingroup_inds, "ingroup_inds(seg, perm|None, preSum, num_unq)");
+    m.def("group_ranks", &group_ranks, "group_ranks(group_inds) -> int64 rank of every element inside its group");
     m.def("dynamic_point_pool", &dynamic_point_pool,
           "dynamic_point_pool(rois, pts, extra_wlh, max_pts_per_box, max_all_pts, rois_batch=None, pts_batch=None)",
           pybind11::arg("rois"), pybind11::arg("pts"), pybind11::arg("extra_wlh"), pybind11::arg("max_pts_per_box"),

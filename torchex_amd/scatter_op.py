@@ -295,13 +295,11 @@ def ingroup_inds(group_inds):
     ``group_inds``: integer ``[N]`` group ids; returns ``[N]`` of the same dtype.
     Ranks ascend with the element index inside a group; the reference hands
     them out with an atomic counter, i.e. in arbitrary order."""
-    ids = group_inds.reshape(-1)
-    if ids.numel() == 0:
+    if group_inds.numel() == 0:
         return torch.zeros_like(group_inds)
-    num_groups = int(ids.max()) + 1          # the reference reads the max on the host too
-    ids32 = ids.int().contiguous()
-    preSum, perm, seg, _, _, _ = scatter_ext.build_plan(ids32, num_groups, scatter_ext.default_heavy_threshold(), None)
-    out = scatter_ext.ingroup_inds(seg, perm, preSum, num_groups)
+    # index preparation of the ids + one rank kernel; the largest id is read on the host (as
+    # the reference does for every call) only when an id reaches the number of elements
+    out = scatter_ext.group_ranks(group_inds)
     return out.to(group_inds.dtype).reshape(group_inds.shape)
 
 
