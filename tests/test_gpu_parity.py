@@ -294,6 +294,26 @@ def test_heavy_threshold_boundary_runs():
     run_case("boundaries_thr32", feats, inv_sorted[p], cnts, heavy_threshold=32)
 
 
+@pytest.mark.parametrize("C", [8, 128])
+def test_heavy_runs_shorter_than_the_long_chunk(C):
+    """Runs of 17..24 rows with the heavy threshold at its minimum (16): every voxel is on the
+    heavy path, the average run is long enough for the forward's 32-position chunk, and such a
+    chunk then meets up to three heavy runs: one more partial than a lane group can park."""
+    g = torch.Generator().manual_seed(61)
+    U = 3000
+    cnts = torch.randint(17, 25, (U,), generator=g)
+    inv_sorted = torch.repeat_interleave(torch.arange(U), cnts)
+    N = int(cnts.sum())
+    assert N >= 8 * U
+    feats = torch.randn((N, C), generator=g)
+    feats[torch.rand((N, C), generator=g) < 0.2] = 1.5          # ties
+    run_case("short_heavy_runs_sorted", feats, inv_sorted, cnts, heavy_threshold=16)
+    p = torch.randperm(N, generator=g)
+    data = run_case("short_heavy_runs_shuffled", feats, inv_sorted[p], cnts, heavy_threshold=16)
+    assert data.num_heavy == U
+    run_case("short_heavy_runs_f16", feats, inv_sorted[p], cnts, heavy_threshold=16, dtype=torch.float16)
+
+
 # ------------------------------------------------- the reference's own test --
 
 def test_reference_test_data_closed_forms(reference_counts):

@@ -79,7 +79,7 @@ __device__ __forceinline__ int ref_rel(int key, int blog2) {  // inverse of ref_
     return (int)((iter << blog2) | ref_prio((unsigned)key >> kIterBits, blog2 - 5));
 }
 
-template <class TR, int VEC, int OP>
+template <class TR, int VEC, int OP, int CHUNK>
 __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     const typename TR::raw *__restrict__ feats, const int *__restrict__ perm,
     const int *__restrict__ seg, const int *__restrict__ slot_of,
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     constexpr bool kRef = OP == TXS_MAX_REFTIE;  // idx[] then holds ref_key, not a row
     extern __shared__ int lds[];
     const int G = kThreads >> lpr_log2;
-    const int T = G * kChunk;
+    const int T = G * CHUNK;
     const int n_seg_s = T + kMargin + 1;  // positions t0-1 .. t0+T+kMargin-1
     int *seg_s = lds;
     int *perm_s = lds + n_seg_s;          // positions t0 .. t0+T+kMargin-1
@@ -147,8 +147,8 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     // Range [la, lb) this lane group reduces: its chunk, minus the tail of an
     // ordinary run that began in an earlier chunk, plus the tail of an ordinary
     // run that begins here and ends later.
-    int la = gi * kChunk + 1;
-    const int lend = min(la + kChunk, N - t0 + 1);
+    int la = gi * CHUNK + 1;
+    const int lend = min(la + CHUNK, N - t0 + 1);
     if (la >= lend) return;
     {
         const int s0 = seg_s[la];
@@ -245,8 +245,24 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                 }
             }
         }
-        // (a third heavy partial in one chunk cannot occur: a heavy run is longer
-        // than a chunk, so a chunk touches at most one at each end)
+        else {
+            // A third heavy partial in one chunk: only a plan whose heavy threshold is below
+            // the chunk has heavy runs short enough for that.  It goes straight to the table.
+            const int slot = slot_of[u];
+            if (slot >= 0) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const size_t o = (size_t)slot * C + col + k;
+                    if constexpr (kMax) {
+                        if (idx[k] >= 0)
+                            atomicMax(scratch + o, ((unsigned long long)ordered_bits((float)acc[k]) << 32) |
+                                                       (unsigned long long)(0xffffffffu - (unsigned)idx[k]));
+                    } else {
+                        unsafeAtomicAdd(reinterpret_cast<float *>(scratch) + o, acc[k]);
+                    }
+                }
+            }
+        }
     };
 
     // Fold one loaded row (position l, voxel sg) into the running reduction.  With
@@ -609,6 +625,16 @@ __global__ __launch_bounds__(kThreads) void scatter_bwd_kernel(
 
 // ------------------------------------------------------------------ launch --
 
+// Sorted positions per lane group of the forward kernel: the long chunk when runs are long on
+// average (fewer heavy-voxel partials to park and merge per row), the short one otherwise
+// (shorter dependent walks, more workgroups).  Between 8 and 64 rows per voxel the long chunk
+// pays for max and for the 2-byte types, whose merges weigh more against their row work; the
+// fp32 sum / mean kernels are faster with the short one there.
+int fwd_chunk_for(long N, long U, bool is_max, int elem) {
+    if (N >= 64 * U) return kChunkLong;
+    return (N >= 8 * U && (is_max || elem == 2)) ? kChunkLong : kChunk;
+}
+
 struct Geometry {
     int vec_bytes;  // bytes one lane moves per row
     int lpr_log2;   // log2(lanes that cover one row slice)
@@ -661,24 +687,20 @@ hipError_t launch_fwd_op(int op, const Geometry &geo, hipStream_t st, const void
     auto s = (unsigned long long *)scratch;
     dim3 blk(kThreads);
     const unsigned lds8 = geo.lds_fwd_idx + 8 * geo.lds_slots;  // 8-byte slot cells for every operator
+#define TXS_FWD_OP(OPC)                                                                           \
+    if (geo.chunk == kChunkLong)                                                                  \
+        scatter_fwd_kernel<TR, VEC, OPC, kChunkLong><<<geo.grid, blk, lds8, st>>>(                \
+            f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);           \
+    else                                                                                          \
+        scatter_fwd_kernel<TR, VEC, OPC, kChunk><<<geo.grid, blk, lds8, st>>>(                    \
+            f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
     switch (op) {
-        case TXS_SUM:
-            scatter_fwd_kernel<TR, VEC, TXS_SUM><<<geo.grid, blk, lds8, st>>>(
-                f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
-            break;
-        case TXS_MEAN:
-            scatter_fwd_kernel<TR, VEC, TXS_MEAN><<<geo.grid, blk, lds8, st>>>(
-                f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
-            break;
-        case TXS_MAX_REFTIE:
-            scatter_fwd_kernel<TR, VEC, TXS_MAX_REFTIE><<<geo.grid, blk, lds8, st>>>(
-                f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
-            break;
-        default:
-            scatter_fwd_kernel<TR, VEC, TXS_MAX><<<geo.grid, blk, lds8, st>>>(
-                f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
-            break;
+        case TXS_SUM: TXS_FWD_OP(TXS_SUM) break;
+        case TXS_MEAN: TXS_FWD_OP(TXS_MEAN) break;
+        case TXS_MAX_REFTIE: TXS_FWD_OP(TXS_MAX_REFTIE) break;
+        default: TXS_FWD_OP(TXS_MAX) break;
     }
+#undef TXS_FWD_OP
     return hipGetLastError();
 }
 
@@ -846,7 +868,7 @@ int scatter_forward_impl(int op, int dtype, const void *feats, const int32_t *un
     const int elem = dtype == TXS_F32 ? 4 : 2;
     hipError_t e = hipSuccess;
     if (N > 0) {
-        Geometry geo = make_geometry(N, C, elem, feats, out, nullptr, is_max, arg, kChunk);
+        Geometry geo = make_geometry(N, C, elem, feats, out, nullptr, is_max, arg, fwd_chunk_for(N, U, is_max, elem));
         if (dtype == TXS_F32)
             e = launch_fwd<F32>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U, ref_log2);
         else if (dtype == TXS_F16)
@@ -915,8 +937,10 @@ int txs_kernel_name(int backward, int op, int dtype, int64_t num_total, int64_t 
                  kOps[op], chunk);
     } else {
         const bool is_max = op == TXS_MAX || op == TXS_MAX_REFTIE;
-        const Geometry geo = make_geometry(num_total, channel, elem, p, p, nullptr, is_max, p, kChunk);
-        snprintf(buf, (size_t)buf_len, "scatter_fwd_kernel<%s,%d,%s>", kTypes[dtype], geo.vec_bytes / elem, kOps[op]);
+        const Geometry geo = make_geometry(num_total, channel, elem, p, p, nullptr, is_max, p,
+                                           fwd_chunk_for(num_total, num_unq, is_max, elem));
+        snprintf(buf, (size_t)buf_len, "scatter_fwd_kernel<%s,%d,%s,%d>", kTypes[dtype], geo.vec_bytes / elem,
+                 kOps[op], geo.chunk);
     }
     return TXS_OK;
 }

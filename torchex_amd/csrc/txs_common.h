@@ -55,6 +55,7 @@ namespace {
 
 constexpr int kThreads = 256;        // 4 wavefronts per workgroup
 constexpr int kChunk = TXS_CHUNK;    // sorted positions per lane group (forward)
+constexpr int kChunkLong = 2 * TXS_CHUNK;  // the same when runs are long on average
 constexpr int kChunkBwdShort = TXS_CHUNK_BWD_SHORT;  // backward kernel, mean run shorter than kChunkBwdLong
 constexpr int kChunkBwdLong = TXS_CHUNK;             // backward kernel, longer runs
 constexpr int kBatchBwd = TXS_BATCH_BWD;
