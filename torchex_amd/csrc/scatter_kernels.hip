@@ -245,9 +245,10 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                 }
             }
         }
-        else {
-            // A third heavy partial in one chunk: only a plan whose heavy threshold is below
-            // the chunk has heavy runs short enough for that.  It goes straight to the table.
+        else if constexpr (CHUNK > kChunk) {
+            // A third heavy partial in one chunk: only the long chunk can meet one, with a plan
+            // whose heavy threshold is below its length (the threshold is never below the
+            // short chunk).  It goes straight to the table.
             const int slot = slot_of[u];
             if (slot >= 0) {
 #pragma unroll
