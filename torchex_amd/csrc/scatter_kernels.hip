@@ -630,10 +630,10 @@ __global__ __launch_bounds__(kThreads) void scatter_bwd_kernel(
 // average (fewer heavy-voxel partials to park and merge per row), the short one otherwise
 // (shorter dependent walks, more workgroups).  Between 8 and 64 rows per voxel the long chunk
 // pays for max and for the 2-byte types, whose merges weigh more against their row work; the
-// fp32 sum / mean kernels are faster with the short one there.
-int fwd_chunk_for(long N, long U, bool is_max, int elem) {
+// fp32 sum / mean kernels and the reference-tie max are faster with the short one there.
+int fwd_chunk_for(long N, long U, int op, int elem) {
     if (N >= 64 * U) return kChunkLong;
-    return (N >= 8 * U && (is_max || elem == 2)) ? kChunkLong : kChunk;
+    return (N >= 8 * U && op != TXS_MAX_REFTIE && (op == TXS_MAX || elem == 2)) ? kChunkLong : kChunk;
 }
 
 struct Geometry {
@@ -869,7 +869,7 @@ int scatter_forward_impl(int op, int dtype, const void *feats, const int32_t *un
     const int elem = dtype == TXS_F32 ? 4 : 2;
     hipError_t e = hipSuccess;
     if (N > 0) {
-        Geometry geo = make_geometry(N, C, elem, feats, out, nullptr, is_max, arg, fwd_chunk_for(N, U, is_max, elem));
+        Geometry geo = make_geometry(N, C, elem, feats, out, nullptr, is_max, arg, fwd_chunk_for(N, U, op, elem));
         if (dtype == TXS_F32)
             e = launch_fwd<F32>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U, ref_log2);
         else if (dtype == TXS_F16)
@@ -939,7 +939,7 @@ int txs_kernel_name(int backward, int op, int dtype, int64_t num_total, int64_t 
     } else {
         const bool is_max = op == TXS_MAX || op == TXS_MAX_REFTIE;
         const Geometry geo = make_geometry(num_total, channel, elem, p, p, nullptr, is_max, p,
-                                           fwd_chunk_for(num_total, num_unq, is_max, elem));
+                                           fwd_chunk_for(num_total, num_unq, op, elem));
         snprintf(buf, (size_t)buf_len, "scatter_fwd_kernel<%s,%d,%s,%d>", kTypes[dtype], geo.vec_bytes / elem,
                  kOps[op], geo.chunk);
     }
