@@ -116,10 +116,22 @@ def cpu_baseline(w, g_mean, g_max):
     tor.step_mean_max(w.feats, w.unq_inv, w.unq_cnts, g_mean, g_max)
     dt1 = time.perf_counter() - t1
     torch.set_num_threads(used)
+    # the C restatement of the reference's algorithm (one core), one step for scale
+    from oracle import c_oracle as orc
+    import numpy as np
+    f32, inv32 = w.feats.numpy(), w.unq_inv.numpy().astype(np.int32)
+    cnt = w.unq_cnts.numpy()
+    t2 = time.perf_counter()
+    orc.mean_from_sum(orc.scatter_sum_f64(f32, inv32, w.U), cnt)
+    orc.mean_backward(g_mean.numpy(), np.maximum(cnt, 1), inv32)
+    _, arg = orc.scatter_max_first(f32, inv32, w.U)
+    orc.max_backward(g_max.numpy(), arg, w.N)
+    dt2 = time.perf_counter() - t2
     return {"value": 2 * w.N / dt, "unit": "points/s", "cores": used,
             "kind": "port", "ms_per_step": dt * 1e3, "single_thread_ms_per_step": dt1 * 1e3,
+            "c_oracle_single_thread_ms_per_step": dt2 * 1e3,
             "sample": f"{iters} full steps (N={w.N}, C={w.C}) of torch.scatter_reduce/index_add/gather on CPU "
-                      f"with {used} threads, then 1 step with 1 thread"}
+                      f"with {used} threads, then 1 step with 1 thread, then 1 step of the C oracle on 1 core"}
 
 
 def instrumented_steps(scatter_ext, f, g_mean, g_max, plan, bplan, steps, warmup):
