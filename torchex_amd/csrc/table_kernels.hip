@@ -413,6 +413,7 @@ TablePlan table_plan(bool backward, int op, int dtype, long N, long C, long U, l
     if (op == TXS_MAX_REFTIE && !backward) return tp;  // the reference's tie key needs voxel order
     if (op == TXS_MAX_REFTIE) op = TXS_MAX;
     if (N <= 0 || C <= 0 || U <= 0) return tp;
+    if (N > 0x7fffffffL - (1L << 16)) return tp;  // the row loops step past the end in 32-bit arithmetic
     // few voxels, many rows each: a partial table per workgroup must stay small next to its rows
     if (N < (long)kTableMinRowsPerVoxel * U || N < 16384) return tp;
     const int elem = dtype == TXS_F32 ? 4 : 2;
