@@ -242,9 +242,9 @@ __device__ __forceinline__ int block_exclusive_scan(int x, int *total) {
 
 int status_of(hipError_t e) { return e == hipSuccess ? TXS_OK : TXS_ERR_LAUNCH; }
 
-// extents are int32 on the device; the margin (more than a tile of 4096 positions plus
-// its look-ahead) keeps position arithmetic from wrapping
-bool fits_i32(int64_t x) { return x >= 0 && x < 2147483647LL - 8192; }
+// extents are int32 on the device; the margin (more than the largest tile, 256 lane groups
+// of 32 positions, plus its look-ahead) keeps position arithmetic from wrapping
+bool fits_i32(int64_t x) { return x >= 0 && x < 2147483647LL - 32768; }
 
 unsigned blocks_for(long n, int per = kThreads) { return (unsigned)((n + per - 1) / per); }
 
