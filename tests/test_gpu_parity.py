@@ -1141,3 +1141,59 @@ def test_plan_with_crowded_buckets_and_the_general_fallback():
         feats = torch.randint(-4, 5, (N, C), generator=g).float()
         data = run_case(name, feats, inv, torch.bincount(inv, minlength=U))
         assert data.max_cnt > crowd // 7 and data.perm is not None
+
+
+def test_element_offsets_beyond_2_to_31():
+    """Maximum sizes: more than 2^31 elements in feats (N * C), in the input gradient and in
+    out / arg (U * C), where the reference's 32-bit `feat_idx * num_dim + dim`
+    (scatter_kernel.cu:115,147) wraps.  The first 16.9 M rows are singletons in shuffled voxel
+    order, so their outputs are the rows themselves; the last 600 k rows, which lie past element
+    2^31, fall into 100 k voxels of their own at the top of the id range and must come out as the
+    same rows do when reduced alone, and that small problem is checked against the oracle."""
+    T = tx()
+    H, TAIL, UT, C = 16_900_000, 600_000, 100_000, 128
+    N, U = H + TAIL, H + UT
+    assert N * C > 2 ** 31 and U * C > 2 ** 31 and H * C > 2 ** 31
+    say(f"[case] offsets beyond 2^31: N={N} U={U} C={C} fp16")
+    g = torch.Generator(device=DEV).manual_seed(31)
+    feats = torch.randn((N, C), generator=g, device=DEV, dtype=torch.float16)
+    head_ids = torch.randperm(H, generator=g, device=DEV)
+    gc = torch.Generator().manual_seed(32)
+    tail_ids = torch.randint(0, UT, (TAIL,), generator=gc)
+    inv = torch.cat([head_ids, tail_ids.to(DEV) + H])
+    cnts = torch.cat([torch.ones(H, dtype=torch.int64), torch.bincount(tail_ids, minlength=UT)]).to(DEV)
+    data = T.ScatterData(inv, cnts)
+    assert data.num_unq == U and data.perm is not None and data.max_cnt == int(cnts.max())
+
+    # the tail alone: a small problem of its own, checked against the oracle
+    ft = feats[H:].contiguous()
+    run_case("tail alone", ft.float().cpu(), tail_ids, torch.bincount(tail_ids, minlength=UT), dtype=torch.float16)
+    dt = T.ScatterData(tail_ids.to(DEV), torch.bincount(tail_ids, minlength=UT).to(DEV))
+    gt = torch.randn((U, C), generator=g, device=DEV, dtype=torch.float16)
+
+    def same_bits(a, b):   # equal bit patterns (NaN included: the mean of an empty voxel)
+        return torch.equal(a.contiguous().view(torch.int16), b.contiguous().view(torch.int16))
+
+    fg = feats.requires_grad_(True)
+    ftg = ft.requires_grad_(True)
+    for name, op in (("sum", T.scatter_sum), ("mean", T.scatter_mean), ("max", T.scatter_max)):
+        say(f"[case] offsets beyond 2^31: {name}")
+        res, res_t = op(fg, data), op(ftg, dt)
+        out, out_t = (res[0], res_t[0]) if name == "max" else (res, res_t)
+        # singletons: the voxel's row itself (sum of one, mean over one, max of one)
+        assert same_bits(out[:H].index_select(0, head_ids), feats[:H].detach()), f"{name}: singleton rows"
+        assert same_bits(out[H:], out_t), f"{name}: voxels of the rows past element 2^31"
+        if name == "max":
+            arg, arg_t = res[1], res_t[1]
+            assert torch.equal(arg[:H].index_select(0, head_ids),
+                               torch.arange(H, device=DEV, dtype=torch.int32)[:, None].expand(H, C))
+            assert torch.equal(arg[H:], torch.where(arg_t >= 0, arg_t + H, arg_t))
+        fg.grad = None
+        ftg.grad = None
+        out.backward(gt)
+        out_t.backward(gt[H:])
+        assert same_bits(fg.grad[H:], ftg.grad), f"{name} backward: rows past element 2^31"
+        # a singleton's gradient row is its voxel's upstream row
+        assert same_bits(fg.grad[:H], gt[:H].index_select(0, head_ids)), f"{name} backward: singleton rows"
+        del res, res_t, out, out_t
+    fg.grad = None
