@@ -225,6 +225,34 @@ int txs_unique_runs(const int32_t *sorted_keys, const int32_t *perm, int64_t num
                     int32_t *preSum, int32_t *stats, void *stream);
 int64_t txs_unique_workspace_len(int64_t num_total);
 
+/* The same triple without a sort, for keys from a bounded grid (a voxelised point cloud: what
+ * test/test_incremental_mask.py:20-26 followed by a torch.unique computes).  An occupancy
+ * map of the key space -- one byte per key set by plain stores, then packed to one bit per
+ * key -- gives every key its dense id: the number of occupied keys below it, i.e. the
+ * unq_inv of torch.unique(keys, return_inverse=True), whose ids ascend with the keys.
+ *   txs_unique_bitmap_count   builds the map and writes the number of distinct keys to
+ *                             stats[NUM_UNQ]; stats[OUT_OF_RANGE] is set if a key is outside
+ *                             [0, key_bound) (the array is not cleared first).
+ *   txs_unique_bitmap_assign  writes unq_inv [num_total] and the ascending unq_keys
+ *                             [up to min(num_total, key_bound)] from the same workspace.
+ * A caller reads NUM_UNQ back while the second call runs, then builds the plan of unq_inv
+ * (txs_plan_build) and takes the counts from its offsets (txs_counts_from_presum).
+ * keys: int32, or int64 when key_is_int64 is non-zero (torch.unique's input as it comes).
+ * The cost grows with key_bound (the map is cleared and read once), so this pays when the
+ * grid is not much larger than the input.  bitmap_ws: int32 workspace of
+ * txs_unique_bitmap_workspace_len(key_bound) entries, 16-byte aligned. */
+int txs_unique_bitmap_count(const void *keys, int key_is_int64, int64_t num_total,
+                            int64_t key_bound, int32_t *bitmap_ws, int32_t *stats, void *stream);
+int txs_unique_bitmap_assign(const void *keys, int key_is_int64, int64_t num_total,
+                             int64_t key_bound, const int32_t *bitmap_ws, int32_t *unq_inv,
+                             int32_t *unq_keys, void *stream);
+int64_t txs_unique_bitmap_workspace_len(int64_t key_bound);
+
+/* unq_cnts[u] = preSum[u + 1] - preSum[u] as int64: the counts torch.unique(...,
+ * return_counts=True) returns, which ScatterData keeps (scatter_op.py:14-17). */
+int txs_counts_from_presum(const int32_t *preSum, int64_t num_unq, int64_t *unq_cnts, void *stream);
+
+
 /* Rank of every element inside its group, from the plan of its group ids:
  * out[row] = sorted position - preSum[group].  Replaces ingroup_inds_launcher
  * (torchex/src/ingroup_inds/ingroup_inds.cpp:14-19, kernel

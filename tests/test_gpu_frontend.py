@@ -94,6 +94,48 @@ def test_from_keys_equals_torch_unique_and_scatter_data(case):
     assert torch.equal(fg.grad, (1.0 / cnt.float()).to(DEV)[inv.to(DEV)].unsqueeze(1).expand(-1, 16))
 
 
+def test_from_keys_occupancy_map_and_sort_agree():
+    """from_keys numbers the keys with an occupancy map of the grid when the grid is not much
+    larger than the input and sorts them otherwise.  The same keys under a small and under a huge
+    bound must give the same triple and plan; int32 and int64 keys alike; the last key of a grid
+    whose size is not a multiple of 32; keys below zero or at the bound raise on both routes."""
+    T = tx()
+    g = torch.Generator().manual_seed(17)
+    N, bound = 200_000, 1_000_003
+    keys = torch.randint(0, bound, (N,), generator=g)
+    keys[:64] = torch.arange(bound - 64, bound)          # the top of the grid, up to bound - 1
+    keys[64:96] = 0
+    unq, inv, cnt = torch.unique(keys, return_inverse=True, return_counts=True)
+    results = []
+    for kdev, b in ((keys.to(DEV), bound), (keys.int().to(DEV), bound), (keys.to(DEV), 2 ** 30),
+                    (keys.int().to(DEV), 2 ** 30)):
+        say(f"[case] from_keys routes: dtype={kdev.dtype} bound={b}")
+        d = T.ScatterData.from_keys(kdev, b)
+        assert torch.equal(d.unq_keys.cpu().long(), unq) and torch.equal(d.unq_inv.cpu().long(), inv)
+        assert torch.equal(d.unq_cnts.cpu().reshape(-1), cnt) and d.unq_cnts.dtype == torch.int64
+        assert d.unq_inv.dtype == torch.int32 and d.unq_keys.dtype == torch.int32
+        assert d.num_unq == unq.shape[0] and d.max_cnt == int(cnt.max())
+        results.append(d)
+    a = results[0]
+    for d in results[1:]:
+        assert torch.equal(d.preSum, a.preSum) and torch.equal(d.perm, a.perm) and torch.equal(d.seg, a.seg)
+        assert torch.equal(d.slot_of, a.slot_of) and torch.equal(d.heavy_ids, a.heavy_ids)
+        assert (d.num_special, d.num_heavy) == (a.num_special, a.num_heavy)
+    for bad_key in (-1, bound):
+        bad = keys.clone()
+        bad[1234] = bad_key
+        for b in (bound, 2 ** 30) if bad_key < 0 else (bound,):
+            with pytest.raises(RuntimeError, match="outside the grid"):
+                T.ScatterData.from_keys(bad.to(DEV), b)
+    # every cell of a small grid occupied, and a grid of one cell
+    full = torch.randperm(4096, generator=g).repeat(3)
+    d = T.ScatterData.from_keys(full.to(DEV), 4096)
+    assert d.num_unq == 4096 and torch.equal(d.unq_keys.cpu().long(), torch.arange(4096))
+    assert torch.equal(d.unq_inv.cpu().long(), full) and int(d.unq_cnts.min()) == 3 == d.max_cnt
+    d = T.ScatterData.from_keys(torch.zeros(500, dtype=torch.int64, device=DEV), 1)
+    assert d.num_unq == 1 and d.max_cnt == 500 and d.perm is None
+
+
 def test_from_points_end_to_end_and_range_check():
     T = tx()
     voxel_size, pc_range = [0.2, 0.2, 0.2], [-75, -75, -2, 75, 75, 4]

@@ -14,6 +14,7 @@
 // PyTorch-ROCm keeps the device type spelled "cuda"; these are its HIP guard
 // and stream accessors for that spelling.
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/HIPEvent.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <algorithm>
@@ -205,16 +206,47 @@ std::tuple<Tensor, Tensor, Tensor> voxel_keys(const Tensor &points, std::vector<
 // scatter plan: one sort, one host synchronisation.
 // returns (unq_keys, unq_inv, unq_cnts, preSum, perm | None, seg, slot_of, heavy_ids, stats)
 std::tuple<Tensor, Tensor, Tensor, Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>>
-unique_plan(const Tensor &keys, int64_t key_bound, int64_t heavy_threshold, const OptTensor &stats_in) {
-    check_i32(keys, "keys");
-    TORCH_CHECK(keys.dim() == 1, "keys must be 1-D");
+unique_plan(const Tensor &keys_in, int64_t key_bound, int64_t heavy_threshold, const OptTensor &stats_in) {
+    check_dev(keys_in, "keys");
+    TORCH_CHECK(keys_in.scalar_type() == at::kInt || keys_in.scalar_type() == at::kLong,
+                "keys must be int32 or int64, got ", keys_in.scalar_type());
+    TORCH_CHECK(keys_in.dim() == 1, "keys must be 1-D");
     TORCH_CHECK(key_bound > 0, "key_bound must be positive");
-    c10::hip::HIPGuardMasqueradingAsCUDA guard(keys.device());
-    const int64_t N = keys.numel();
-    void *st = cur_stream(keys);
-    Tensor stats = stats_in.has_value() ? *stats_in : at::zeros({TXS_STATS_LEN}, keys.options());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(keys_in.device());
+    const int64_t N = keys_in.numel();
+    void *st = cur_stream(keys_in);
+    const auto i32 = keys_in.options().dtype(at::kInt);
+    Tensor stats = stats_in.has_value() ? *stats_in : at::zeros({TXS_STATS_LEN}, i32);
     check_i32(stats, "stats");
     TORCH_CHECK(stats.numel() == TXS_STATS_LEN, "stats must have TXS_STATS_LEN entries");
+    // Keys from a grid that is not much larger than the input: dense ids from an occupancy
+    // map (no sort of the keys), then the index preparation of those ids.  `stats` is read
+    // twice: the number of distinct keys, which sizes the plan (fetched while the ids are
+    // still being written), and the plan's own figures.
+    if (N > 0 && key_bound <= (int64_t(1) << 28) && key_bound <= 64 * N) {
+        const int is64 = keys_in.scalar_type() == at::kLong;
+        Tensor inv = at::empty({N}, i32), unq = at::empty({std::min(N, key_bound)}, i32);
+        Tensor bws = at::empty({txs_unique_bitmap_workspace_len(key_bound)}, i32);
+        check_status(txs_unique_bitmap_count(keys_in.data_ptr(), is64, N, key_bound, i32w(bws), i32w(stats), st),
+                     "unique_bitmap_count");
+        Tensor h = at::empty({TXS_STATS_LEN}, stats.options().device(at::kCPU).pinned_memory(true));
+        h.copy_(stats, /*non_blocking=*/true);
+        at::cuda::CUDAEvent counted;
+        counted.record(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(keys_in.device().index()));
+        check_status(txs_unique_bitmap_assign(keys_in.data_ptr(), is64, N, key_bound, i32p(bws), i32w(inv), i32w(unq), st),
+                     "unique_bitmap_assign");
+        counted.synchronize();
+        TORCH_CHECK(h.data_ptr<int32_t>()[TXS_STAT_OUT_OF_RANGE] == 0,
+                    "keys (or points) outside the grid: keys must be in [0, ", key_bound, ")");
+        const int64_t U = h.data_ptr<int32_t>()[TXS_STAT_NUM_UNQ];
+        auto [preSum, perm_out, seg, slot_of, heavy_ids, hs] = build_plan(inv, U, heavy_threshold, std::nullopt, false);
+        Tensor cnts = at::empty({U}, keys_in.options().dtype(at::kLong));
+        check_status(txs_counts_from_presum(i32p(preSum), U, U ? cnts.data_ptr<int64_t>() : nullptr, st),
+                     "counts_from_presum");
+        hs[TXS_STAT_NUM_UNQ] = U;
+        return {unq.narrow(0, 0, U), inv, cnts, preSum, perm_out, seg, slot_of, heavy_ids, hs};
+    }
+    const Tensor keys = keys_in.scalar_type() == at::kInt ? keys_in : keys_in.to(at::kInt);
     Tensor seg = empty_i32(N, keys), perm = empty_i32(N, keys), inv = empty_i32(N, keys);
     Tensor unq = empty_i32(N, keys), preSum = empty_i32(N + 1, keys);
     Tensor slot_of = empty_i32(N, keys), heavy_all = empty_i32(N, keys);

@@ -118,7 +118,7 @@ class ScatterData:
             heavy_threshold = scatter_ext.default_heavy_threshold()
         self.heavy_threshold = int(heavy_threshold)
         flat = keys.reshape(-1)
-        if flat.dtype != torch.int32:
+        if flat.dtype not in (torch.int32, torch.int64):
             flat = flat.int()
         flat = flat.contiguous()
         (self.unq_keys, self.unq_inv, cnts, self.preSum, self.perm, self.seg, self.slot_of,
