@@ -1197,3 +1197,47 @@ def test_element_offsets_beyond_2_to_31():
         assert same_bits(fg.grad[:H], gt[:H].index_select(0, head_ids)), f"{name} backward: singleton rows"
         del res, res_t, out, out_t
     fg.grad = None
+
+
+def test_python_function_classes_and_module_level_operators_agree():
+    """`scatter_sum / scatter_mean / scatter_max` run an autograd node written in C++; the
+    `Scatter*Function` classes with the reference's names (scatter_op.py:24-111) are Python
+    `autograd.Function`s over the same launches.  Same outputs, same gradients, `arg` carries
+    no gradient on either, a call under `no_grad` records nothing, and a gradient that reaches
+    only `arg`'s partner of a tuple still flows."""
+    T = tx()
+    from torchex_amd import scatter_op as so
+    w = workloads.lidar_sweep(N=60_000, C=48, seed=21)
+    data = T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV))
+    g = workloads.upstream_grad(w.U, w.C, 5).to(DEV)
+    for fast, cls in ((T.scatter_sum, so.ScatterSumFunction), (T.scatter_mean, so.ScatterMeanFunction),
+                      (T.scatter_max, so.ScatterMaxFunction)):
+        fa = w.feats.to(DEV).requires_grad_(True)
+        fb = w.feats.to(DEV).requires_grad_(True)
+        ra, rb = fast(fa, data), cls.apply(fb, data)
+        if cls is so.ScatterMaxFunction:
+            assert isinstance(ra, tuple) and len(ra) == 2
+            assert torch.equal(ra[1], rb[1]) and ra[1].dtype == torch.int32
+            assert not ra[1].requires_grad and not rb[1].requires_grad
+            ra, rb = ra[0], rb[0]
+        assert ra.requires_grad and ra.grad_fn is not None
+        assert torch.equal(ra, rb)
+        ra.backward(g)
+        rb.backward(g)
+        assert torch.equal(fa.grad, fb.grad)
+        with torch.no_grad():
+            rn = fast(fa, data)
+        rn = rn[0] if isinstance(rn, tuple) else rn
+        assert not rn.requires_grad and torch.equal(rn, ra)
+    # part of a larger graph, twice through the same ScatterData
+    f = w.feats.to(DEV).requires_grad_(True)
+    mx, _ = T.scatter_max(f * 2.0, data)
+    loss = (mx * g).sum() + (T.scatter_mean(f, data) * g).sum()
+    loss.backward()
+    f2 = w.feats.to(DEV).requires_grad_(True)
+    mx2, _ = so.ScatterMaxFunction.apply(f2 * 2.0, data)
+    ((mx2 * g).sum() + (so.ScatterMeanFunction.apply(f2, data) * g).sum()).backward()
+    assert torch.equal(f.grad, f2.grad)
+    # features that need no gradient: no node at all
+    out = T.scatter_sum(w.feats.to(DEV), data)
+    assert not out.requires_grad and out.grad_fn is None

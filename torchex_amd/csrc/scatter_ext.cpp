@@ -436,7 +436,7 @@ int check_path(int64_t path) {
 
 void run_forward(int op, const Tensor &feats, const OptTensor &unq_inv, const OptTensor &perm, const Tensor &seg,
                  const Tensor &preSum, const Tensor &slot_of, const Tensor &heavy_ids, int64_t num_heavy,
-                 Tensor &scratch, Tensor &out, OptTensor &arg, int64_t max_cnt, int path) {
+                 Tensor &scratch, Tensor &out, OptTensor &arg, int64_t max_cnt, int path, bool holds_gil = true) {
     const int64_t N = feats.size(0), C = feats.size(1), U = preSum.numel() - 1;
     const int64_t S = heavy_ids.numel();
     TORCH_CHECK(scratch.dim() == 1, "scratch must be 1-D (ScatterData.scratch(channel))");
@@ -450,24 +450,29 @@ void run_forward(int op, const Tensor &feats, const OptTensor &unq_inv, const Op
     TORCH_CHECK(out.size(0) == U && out.size(1) == C, "out must be [num_unq, channel]");
     const int dt = dtype_code(feats, "feats");
     void *st = cur_stream(feats);
+    auto launch = [&]() {
+        return txs_scatter_forward(op, dt, feats.data_ptr(), opt_i32p(unq_inv), opt_i32p(perm), i32p(seg),
+                                   i32p(preSum), i32p(slot_of), i32p(heavy_ids), S, num_heavy,
+                                   scratch.numel() ? scratch.data_ptr() : nullptr, scratch.numel(), out.data_ptr(),
+                                   arg.has_value() ? arg->data_ptr<int32_t>() : nullptr, N, C, U, max_cnt, path,
+                                   st);
+    };
     int rc;
-    {
+    if (holds_gil) {
         pybind11::gil_scoped_release nogil;
-        rc = txs_scatter_forward(op, dt, feats.data_ptr(), opt_i32p(unq_inv), opt_i32p(perm), i32p(seg),
-                                 i32p(preSum), i32p(slot_of), i32p(heavy_ids), S, num_heavy,
-                                 scratch.numel() ? scratch.data_ptr() : nullptr, scratch.numel(), out.data_ptr(),
-                                 arg.has_value() ? arg->data_ptr<int32_t>() : nullptr, N, C, U, max_cnt, path,
-                                 st);
+        rc = launch();
+    } else {
+        rc = launch();
     }
     check_status(rc, "scatter_forward");
 }
 
 // forward(op, feats, unq_inv|None, perm|None, seg, preSum, slot_of, heavy_ids, num_heavy, scratch, max_cnt,
 //         path=0) -> (out, arg|None)
-std::tuple<Tensor, OptTensor> forward(int64_t op, const Tensor &feats, const OptTensor &unq_inv,
-                                      const OptTensor &perm, const Tensor &seg, const Tensor &preSum,
-                                      const Tensor &slot_of, const Tensor &heavy_ids, int64_t num_heavy,
-                                      Tensor scratch, int64_t max_cnt, int64_t path) {
+std::tuple<Tensor, OptTensor> forward_impl(int64_t op, const Tensor &feats, const OptTensor &unq_inv,
+                                           const OptTensor &perm, const Tensor &seg, const Tensor &preSum,
+                                           const Tensor &slot_of, const Tensor &heavy_ids, int64_t num_heavy,
+                                           Tensor scratch, int64_t max_cnt, int64_t path, bool holds_gil) {
     check_dev(feats, "feats");
     TORCH_CHECK(feats.dim() == 2, "feats must be [num_total, channel]");
     check_i32(seg, "seg");
@@ -485,13 +490,22 @@ std::tuple<Tensor, OptTensor> forward(int64_t op, const Tensor &feats, const Opt
     OptTensor arg;
     if (op == TXS_MAX || op == TXS_MAX_REFTIE) arg = at::empty({U, C}, feats.options().dtype(at::kInt));
     run_forward((int)op, feats, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_heavy, scratch, out, arg, max_cnt,
-                check_path(path));
+                check_path(path), holds_gil);
     return {out, arg};
 }
 
+std::tuple<Tensor, OptTensor> forward(int64_t op, const Tensor &feats, const OptTensor &unq_inv,
+                                      const OptTensor &perm, const Tensor &seg, const Tensor &preSum,
+                                      const Tensor &slot_of, const Tensor &heavy_ids, int64_t num_heavy,
+                                      Tensor scratch, int64_t max_cnt, int64_t path) {
+    return forward_impl(op, feats, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_heavy, std::move(scratch),
+                        max_cnt, path, /*holds_gil=*/true);
+}
+
 // backward(op, grad_out, arg|None, unq_inv|None, perm|None, seg, preSum, num_total, path=0) -> grad_in
-Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const OptTensor &unq_inv,
-                const OptTensor &perm, const Tensor &seg, const Tensor &preSum, int64_t num_total, int64_t path) {
+Tensor backward_impl(int64_t op, const Tensor &grad_out, const OptTensor &arg, const OptTensor &unq_inv,
+                     const OptTensor &perm, const Tensor &seg, const Tensor &preSum, int64_t num_total, int64_t path,
+                     bool holds_gil) {
     check_dev(grad_out, "grad_out");
     TORCH_CHECK(grad_out.dim() == 2, "grad_out must be [num_unq, channel]");
     check_i32(seg, "seg");
@@ -514,14 +528,78 @@ Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const 
     const int pth = check_path(path);
     Tensor gin = at::empty({N, C}, grad_out.options());
     void *st = cur_stream(grad_out);
+    auto launch = [&]() {
+        return txs_scatter_backward((int)op, dt, grad_out.data_ptr(), opt_i32p(arg), opt_i32p(unq_inv),
+                                    opt_i32p(perm), i32p(seg), i32p(preSum), gin.data_ptr(), N, C, U, pth, st);
+    };
     int rc;
-    {
+    if (holds_gil) {
         pybind11::gil_scoped_release nogil;
-        rc = txs_scatter_backward((int)op, dt, grad_out.data_ptr(), opt_i32p(arg), opt_i32p(unq_inv),
-                                  opt_i32p(perm), i32p(seg), i32p(preSum), gin.data_ptr(), N, C, U, pth, st);
+        rc = launch();
+    } else {
+        rc = launch();
     }
     check_status(rc, "scatter_backward");
     return gin;
+}
+
+Tensor backward(int64_t op, const Tensor &grad_out, const OptTensor &arg, const OptTensor &unq_inv,
+                const OptTensor &perm, const Tensor &seg, const Tensor &preSum, int64_t num_total, int64_t path) {
+    return backward_impl(op, grad_out, arg, unq_inv, perm, seg, preSum, num_total, path, /*holds_gil=*/true);
+}
+
+// The operators as one autograd node written in C++ (what ScatterSumFunction /
+// ScatterMeanFunction / ScatterMaxFunction of scatter_op.py:24-111 are in Python): the node's
+// forward and backward call the same launch functions, without the Python-side
+// autograd.Function machinery, which costs more host time per call than a small input's
+// kernels take on the GPU.  The gradient goes to feats only; arg is not differentiable.
+struct ScatterNode : public torch::autograd::Function<ScatterNode> {
+    static torch::autograd::variable_list forward(torch::autograd::AutogradContext *ctx, const Tensor &feats,
+                                                  int64_t op, const OptTensor &unq_inv, const OptTensor &perm,
+                                                  const Tensor &seg, const Tensor &preSum, const Tensor &slot_of,
+                                                  const Tensor &heavy_ids, int64_t num_heavy, const Tensor &scratch,
+                                                  int64_t max_cnt, int64_t path) {
+        auto [out, arg] = forward_impl(op, feats, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_heavy, scratch,
+                                       max_cnt, path, /*holds_gil=*/PyGILState_Check() != 0);
+        ctx->saved_data["op"] = op;
+        ctx->saved_data["path"] = path;
+        ctx->saved_data["num_total"] = feats.size(0);
+        const Tensor none;
+        ctx->save_for_backward({arg.has_value() ? *arg : none, unq_inv.has_value() ? *unq_inv : none,
+                                perm.has_value() ? *perm : none, seg, preSum});
+        ctx->set_materialize_grads(false);  // no zero tensor for the integer output's gradient slot
+        if (arg.has_value()) {
+            ctx->mark_non_differentiable({*arg});
+            return {out, *arg};
+        }
+        return {out};
+    }
+
+    static torch::autograd::variable_list backward(torch::autograd::AutogradContext *ctx,
+                                                   torch::autograd::variable_list grads) {
+        torch::autograd::variable_list result(12);  // one slot per forward argument; only feats gets a gradient
+        if (grads.empty() || !grads[0].defined()) return result;
+        const auto saved = ctx->get_saved_variables();
+        auto opt = [](const Tensor &t) -> OptTensor { return t.defined() ? OptTensor(t) : std::nullopt; };
+        const int64_t op = ctx->saved_data["op"].toInt();
+        // the engine's worker threads run this without the interpreter lock
+        result[0] = backward_impl(op, grads[0].contiguous(), opt(saved[0]), opt(saved[1]), opt(saved[2]), saved[3],
+                                  saved[4], ctx->saved_data["num_total"].toInt(), ctx->saved_data["path"].toInt(),
+                                  /*holds_gil=*/PyGILState_Check() != 0);
+        return result;
+    }
+};
+
+// scatter(op, feats, <plan arguments of forward>) -> (out, arg | None), differentiable in feats
+std::tuple<Tensor, OptTensor> scatter_autograd(int64_t op, const Tensor &feats, const OptTensor &unq_inv,
+                                               const OptTensor &perm, const Tensor &seg, const Tensor &preSum,
+                                               const Tensor &slot_of, const Tensor &heavy_ids, int64_t num_heavy,
+                                               const Tensor &scratch, int64_t max_cnt, int64_t path) {
+    auto res = ScatterNode::apply(feats, op, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_heavy, scratch,
+                                  max_cnt, path);
+    OptTensor arg;
+    if (res.size() > 1) arg = res[1];
+    return {res[0], arg};
 }
 
 // ---- the reference module's three functions (scatter.cpp:20-64) ------------
@@ -694,6 +772,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("csr_plan_cache_size", &csr_plan_cache_size, "number of plans currently kept for sum/max over CSR offsets");
     m.def("forward", &forward,
           "forward(op, feats, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_heavy, scratch, max_cnt, path=0)",
+          pybind11::arg("op"), pybind11::arg("feats"), pybind11::arg("unq_inv"), pybind11::arg("perm"),
+          pybind11::arg("seg"), pybind11::arg("preSum"), pybind11::arg("slot_of"), pybind11::arg("heavy_ids"),
+          pybind11::arg("num_heavy"), pybind11::arg("scratch"), pybind11::arg("max_cnt"), pybind11::arg("path") = 0);
+    m.def("scatter", &scatter_autograd,
+          "scatter(op, feats, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_heavy, scratch, max_cnt, path=0) -> "
+          "(out, arg|None): forward(...) as an autograd node, differentiable in feats",
           pybind11::arg("op"), pybind11::arg("feats"), pybind11::arg("unq_inv"), pybind11::arg("perm"),
           pybind11::arg("seg"), pybind11::arg("preSum"), pybind11::arg("slot_of"), pybind11::arg("heavy_ids"),
           pybind11::arg("num_heavy"), pybind11::arg("scratch"), pybind11::arg("max_cnt"), pybind11::arg("path") = 0);

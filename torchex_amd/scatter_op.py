@@ -303,7 +303,30 @@ def ingroup_inds(group_inds):
     return out.to(group_inds.dtype).reshape(group_inds.shape)
 
 
-scatter_sum = ScatterSumFunction.apply
-scatter_mean = ScatterMeanFunction.apply
-scatter_max = ScatterMaxFunction.apply
+# The reference binds ``scatter_sum = ScatterSumFunction.apply`` etc. (scatter_op.py:138-141).
+# Same call form and results here; the autograd node behind these three is the C++ one in
+# scatter_ext (``scatter_ext.scatter``), which spares the host the Python-side
+# ``autograd.Function`` machinery on every call -- on small inputs that costs more than the
+# kernels.  The ``*Function`` classes above stay usable through ``.apply``.
+
+def scatter_sum(feats, data):
+    """``scatter_sum(feats, data) -> [num_unq, channel]`` (``scatter_op.py:27-50``)."""
+    _check_feats(feats, data)
+    return scatter_ext.scatter(_SUM, feats, *data.forward_args(feats.shape[1]))[0]
+
+
+def scatter_mean(feats, data):
+    """``scatter_mean(feats, data) -> [num_unq, channel]`` (``scatter_op.py:56-78``)."""
+    _check_feats(feats, data)
+    return scatter_ext.scatter(_MEAN, feats, *data.forward_args(feats.shape[1]))[0]
+
+
+def scatter_max(feats, data):
+    """``scatter_max(feats, data) -> (out, arg)`` (``scatter_op.py:84-111``); the tie rule is
+    ``data.max_tie_rule`` as described for ``ScatterMaxFunction``."""
+    _check_feats(feats, data)
+    op = scatter_ext.MAX_REFTIE if data.max_tie_rule == "reference" else _MAX
+    return scatter_ext.scatter(op, feats, *data.forward_args(feats.shape[1]))
+
+
 getPreSum = GetPreSumFunction.apply
