@@ -1128,11 +1128,12 @@ def test_table_kernels_special_values_and_grouped_rows():
 
 def test_plan_with_crowded_buckets_and_the_general_fallback():
     """Index preparation splits the ids into buckets of consecutive voxels.  A bucket with far
-    more rows than the others is shared by several workgroups; one that holds more than 262,144
-    rows sends the whole plan to the general radix passes.  Both give the same plan as the oracle."""
+    more rows than the others is cut into slices of 2048 rows, one workgroup each; beyond 64
+    slices the slices get longer; a bucket of more than 262,144 rows sends the whole plan to the
+    general radix passes.  All give the same plan as the oracle."""
     g = torch.Generator().manual_seed(13)
     U, C = 5000, 8                      # 13 bits of id: buckets of 32 consecutive voxels
-    for name, crowd in (("shared bucket", 100_000), ("giant bucket", 300_000)):
+    for name, crowd in (("shared bucket", 100_000), ("long slices", 200_000), ("giant bucket", 300_000)):
         N = crowd + 120_000
         inv = torch.randint(0, U, (N,), generator=g)
         hot = torch.randperm(N, generator=g)[:crowd]

@@ -337,26 +337,31 @@ __global__ void seg_from_presum_kernel(const int *__restrict__ preSum, long n, i
 
 // ------------------------------------------------ two-level plan (bucket sort) --
 //
-// For up to 2^22 voxels the whole index preparation is three kernels and a scan:
-//   (1) bucket_hist_kernel: per tile of 8192 rows, the histogram of the HIGH digit of the
+// For up to 2^22 voxels the whole index preparation is four kernels and a scan:
+//   (1) bucket_hist_kernel: per tile of 2048 - 8192 rows, the histogram of the HIGH digit of the
 //       voxel id (the "bucket") and the tile's order / range flags;
 //   (2) exclusive scan of the digit-major histogram;
 //   (3) bucket_scatter_kernel: flags of the whole input, bucket boundaries, and the stable
 //       scatter of (id, row) pairs by bucket (wave-ballot ranking);
-//   (4) bucket_plan_kernel: counting sort of every bucket by the LOW digit (<= 11 bits) in
-//       LDS, which at the same time yields the bucket's slice of everything else the plan
-//       holds: CSR offsets, per-voxel counts (checked against the caller's), the
-//       special-voxel table and its slots, max_cnt, and the flagged per-position ids
-//       written next to the permutation.  A bucket of more than 8192 rows is shared by up
-//       to 16 workgroups: each counts the whole bucket (LDS integer atomics) and the rows
-//       in front of its own slice, then places its slice.
+//   (4) bucket_count_kernel: a bucket is cut into slices of 2048 rows (at most 64, longer ones
+//       beyond), one workgroup per slice; each counts its slice's rows per voxel (LOW digit,
+//       <= 11 bits) in LDS and writes the counts out;
+//   (5) bucket_plan_kernel: the same workgroups add up the counts of their bucket's slices
+//       (a voxel's count, and its rows in the slices in front), which at the same time yields
+//       the bucket's share of everything else the plan holds: CSR offsets, per-voxel counts
+//       (checked against the caller's), the special-voxel table and its slots, max_cnt; then
+//       each places its slice by the low digit, stably, writing the flagged per-position ids
+//       next to the permutation.
+// (Measured against one kernel in which every workgroup of a bucket counted the whole bucket:
+// 1M ids of a voxelised sweep 67 -> 63 us, of its pillars 64 -> 57 us, 200k ids 38 -> 41 us
+// (one launch more), and 1.25M ids of which 250k fall into 900 neighbouring voxels 198 -> 101 us.)
 // Ids of at most 11 bits need no low digit: (3) already gives the final order, and the
 // elementwise kernels used by the general sequence finish the plan.
 // Measured alternatives (1M ids of 19 bits, 0.13 ms per plan as built): an 11-bit bucket digit
 // makes the scatter write 16-byte runs and costs 30 us instead of 20; folding the scan into
 // the scatter (every workgroup adding up the tile histograms itself) saves two launches but
 // costs more than it saves from about 100 tiles on; per-voxel instead of per-row offset
-// bookkeeping in (4) makes no difference.
+// bookkeeping in (5) makes no difference.
 
 #ifndef TXS_BUCKET_HIGH_BITS
 #define TXS_BUCKET_HIGH_BITS 9
@@ -381,7 +386,10 @@ constexpr int kBktItems = TXS_BKT_ITEMS;
 constexpr int kBktChunk = kThreads * kBktItems;        // 4096 rows per placement round
 constexpr int kBktWaves = kThreads / 64;
 constexpr int kBktSlice = TXS_BKT_SLICE_CHUNKS * kBktChunk;  // rows one workgroup places
-constexpr int kBktMaxSlices = 16;                      // workgroups per bucket at most
+#ifndef TXS_BKT_MAX_SLICES
+#define TXS_BKT_MAX_SLICES 64
+#endif
+constexpr int kBktMaxSlices = TXS_BKT_MAX_SLICES;      // workgroups per bucket at most
 constexpr long kBktGiant = 262144;                     // rows in one bucket beyond which the general sequence runs
 constexpr int kFlagUnsorted = 1, kFlagOutOfRange = 2;
 
@@ -538,33 +546,53 @@ __global__ __launch_bounds__(kHistThreads) void bucket_scatter_kernel(
     }
 }
 
-// Workgroup g serves slice j of bucket b; (b, j) follows from the bucket sizes.
-__global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
-    const int *__restrict__ inv, const int *__restrict__ pairs1, long n, int U,
-    int low_bits, int high_bins, const int *__restrict__ bucket_start, int heavy_threshold,
-    const long long *__restrict__ unq_cnts, int *__restrict__ perm, int *__restrict__ seg,
-    int *__restrict__ preSum, int *__restrict__ slot_of, int *__restrict__ heavy_ids,
-    int *__restrict__ stats) {
-    extern __shared__ int wc[];  // [kBktWaves][low_bins], tot[low_bins], off[low_bins]
-    __shared__ int s_pick[2], s_red[kBktWaves], s_bad[kBktWaves];
-    const int low_bins = 1 << low_bits;
-    int *tot = wc + kBktWaves * low_bins;
-    int *off = tot + low_bins;
-    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const unsigned long long lanes_below = (1ull << lane) - 1ull;
-    if (stats[TXS_STAT_NEED_GENERAL] != 0) return;
+// Rows of bucket b that slice j of it covers.  A bucket is cut into slices of kBktSlice rows,
+// at most kBktMaxSlices of them (longer slices beyond that).
+struct BucketSlice {
+    long s, e;        // the bucket's rows [s, e) in bucket order
+    long my_s, my_e;  // the slice's rows
+    int nsl;          // slices of the bucket
+};
+__device__ __forceinline__ int slices_of(long cnt_b) {
+    return (int)min((long)kBktMaxSlices, max(1L, (cnt_b + kBktSlice - 1) / kBktSlice));
+}
+__device__ __forceinline__ BucketSlice bucket_slice(long s, long e, int j) {
+    BucketSlice r;
+    r.s = s;
+    r.e = e;
+    const long nb = r.e - r.s;
+    r.nsl = slices_of(nb);
+    long slice = kBktSlice;
+    if (nb > (long)kBktMaxSlices * kBktSlice)
+        slice = ((nb + kBktMaxSlices - 1) / kBktMaxSlices + kBktChunk - 1) / kBktChunk * kBktChunk;
+    r.my_s = r.s + (long)j * slice;
+    r.my_e = min(r.e, r.my_s + slice);
+    return r;
+}
 
-    // ---- which (bucket, slice) is this workgroup's?
+// Workgroup g serves slice j of bucket b; (b, j) follows from the bucket sizes and is kept with
+// the bucket's bounds in wg_pick[g] = (b, j, start, end) (b = -1: no work) for the kernel that
+// follows, which so learns its work from one load.  Each workgroup
+// counts the rows of ITS slice per voxel (low digit) and writes the counts to part_hist[g][*]:
+// the slices of a bucket sit in consecutive workgroups, so the next kernel gets a voxel's count in
+// the whole bucket, and in the slices in front of its own, from at most kBktMaxSlices short
+// reads instead of every workgroup of a crowded bucket counting all of its rows.
+__global__ __launch_bounds__(kThreads) void bucket_count_kernel(
+    const int *__restrict__ inv, const int *__restrict__ pairs1, long n, int U, int low_bits, int high_bins,
+    const int *__restrict__ bucket_start, const int *__restrict__ stats, int4 *__restrict__ wg_pick,
+    int *__restrict__ part_hist) {
+    extern __shared__ int cnt_s[];  // [low_bins]
+    __shared__ int s_pick[2];
+    const int low_bins = 1 << low_bits;
+    if (stats[TXS_STAT_NEED_GENERAL] != 0) return;
     {
         if (threadIdx.x == 0) s_pick[0] = -1;
         int carried = 0;
         for (int bb0 = 0; bb0 < high_bins; bb0 += kThreads) {
             const int bb = bb0 + (int)threadIdx.x;
             int nsl = 0;
-            if (bb < high_bins && ((long)bb << low_bits) < (long)U) {
-                const long cnt_b = (long)bucket_start[bb + 1] - bucket_start[bb];
-                nsl = (int)min((long)kBktMaxSlices, max(1L, (cnt_b + kBktSlice - 1) / kBktSlice));
-            }
+            if (bb < high_bins && ((long)bb << low_bits) < (long)U)
+                nsl = slices_of((long)bucket_start[bb + 1] - bucket_start[bb]);
             int total;
             const int first = carried + block_exclusive_scan(nsl, &total);  // (synchronises the workgroup)
             if ((int)blockIdx.x >= first && (int)blockIdx.x < first + nsl) {
@@ -576,23 +604,84 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
         __syncthreads();
     }
     const int b = s_pick[0], j = s_pick[1];
+    if (b < 0) {
+        if (threadIdx.x == 0) wg_pick[blockIdx.x] = make_int4(-1, 0, 0, 0);
+        return;
+    }
+    const int u_lo = b << low_bits;
+    const bool packed = stats[TXS_STAT_UNSORTED] != 0;
+    const int *keys = packed ? pairs1 : inv;
+    const BucketSlice sl = bucket_slice(bucket_start[b], bucket_start[b + 1], j);
+    if (threadIdx.x == 0) wg_pick[blockIdx.x] = make_int4(b, j, (int)sl.s, (int)sl.e);
+    for (int k = threadIdx.x; k < low_bins; k += kThreads) cnt_s[k] = 0;
+    __syncthreads();
+    for (long i0 = sl.my_s; i0 < sl.my_e; i0 += (long)kThreads * kBktItems) {
+        int v[kBktItems];
+#pragma unroll
+        for (int it = 0; it < kBktItems; ++it) {
+            const long i = i0 + (long)it * kThreads + threadIdx.x;
+            v[it] = i < sl.my_e ? kread(keys, i, packed) : -1;
+        }
+#pragma unroll
+        for (int it = 0; it < kBktItems; ++it) {
+            const int d = v[it] - u_lo;
+            if (v[it] >= 0 && (unsigned)d < (unsigned)low_bins) atomicAdd(&cnt_s[d], 1);
+        }
+    }
+    __syncthreads();
+    int *mine = part_hist + (long)blockIdx.x * low_bins;
+    for (int k = threadIdx.x; k < low_bins; k += kThreads) mine[k] = cnt_s[k];
+}
+
+__global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
+    const int *__restrict__ inv, const int *__restrict__ pairs1, long n, int U,
+    int low_bits, int high_bins, const int *__restrict__ bucket_start, int heavy_threshold,
+    const long long *__restrict__ unq_cnts, int *__restrict__ perm, int *__restrict__ seg,
+    int *__restrict__ preSum, int *__restrict__ slot_of, int *__restrict__ heavy_ids,
+    int *__restrict__ stats, const int4 *__restrict__ wg_pick, const int *__restrict__ part_hist) {
+    extern __shared__ int wc[];  // [kBktWaves][low_bins], tot[low_bins], off[low_bins]
+    __shared__ int s_red[kBktWaves], s_bad[kBktWaves];
+    const int low_bins = 1 << low_bits;
+    int *tot = wc + kBktWaves * low_bins;
+    int *off = tot + low_bins;
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const unsigned long long lanes_below = (1ull << lane) - 1ull;
+    if (stats[TXS_STAT_NEED_GENERAL] != 0) return;
+    (void)high_bins;
+    const int4 pick = wg_pick[blockIdx.x];
+    const int b = pick.x, j = pick.y;
     if (b < 0) return;
     const int u_lo = b << low_bits;
     const int u_hi = min(U, u_lo + low_bins);
     const bool unsorted = stats[TXS_STAT_UNSORTED] != 0;
     const bool packed = unsorted;
-    const int *keys = unsorted ? pairs1 : inv;
-    const long s = bucket_start[b];
-    const long e = bucket_start[b + 1];
-    const long nb = e - s;
-    long slice = kBktSlice;
-    if (nb > (long)kBktMaxSlices * kBktSlice)
-        slice = ((nb + kBktMaxSlices - 1) / kBktMaxSlices + kBktChunk - 1) / kBktChunk * kBktChunk;
-    const long my_s = s + (long)j * slice;
-    const long my_e = min(e, my_s + slice);
+    const BucketSlice sl = bucket_slice(pick.z, pick.w, j);
+    const long s = sl.s, e = sl.e, my_s = sl.my_s, my_e = sl.my_e;
 
-    // the caller's counts of this bucket's voxels (first slice only) are fetched now and
-    // compared once the kernel's own counts are complete
+    // Everything the workgroup reads from memory is requested here, in one go: the first
+    // round of the slice's rows, the caller's counts of this bucket's voxels (first slice
+    // only; compared once the kernel's own counts are complete), and the per-slice counts.
+    auto load_round = [&](long c0, int (&key)[kBktItems], int (&row)[kBktItems]) {
+        const long wbase = c0 + (long)w * (64 * kBktItems);
+#pragma unroll
+        for (int it = 0; it < kBktItems; ++it) {
+            const long i = wbase + (long)it * 64 + lane;
+            int v = -1;
+            row[it] = (int)i;
+            if (i < my_e) {
+                if (packed) {
+                    const int2 kr = reinterpret_cast<const int2 *>(pairs1)[i];
+                    v = kr.x;
+                    row[it] = kr.y;
+                } else {
+                    v = inv[i];
+                }
+            }
+            key[it] = (i < my_e && (unsigned)(v - u_lo) < (unsigned)low_bins) ? v : -1;
+        }
+    };
+    int key0[kBktItems], row0[kBktItems];
+    load_round(my_s, key0, row0);
     constexpr int kCntPer = (1 << kBucketLowBitsMax) / kThreads;
     long long given[kCntPer];
     const bool check_counts = j == 0 && unq_cnts != nullptr;
@@ -603,48 +692,30 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
             given[k] = (d < low_bins && u_lo + d < u_hi) ? unq_cnts[u_lo + d] : -1;
         }
     }
-    // ---- counts of the bucket's voxels, and of the rows in front of this slice
+    // ---- counts of the bucket's voxels, and of the rows in front of this slice: sums over the
+    // per-slice counts of the bucket's workgroups (blockIdx.x - j is the bucket's first), eight
+    // loads in flight per thread
     for (int k = threadIdx.x; k < (kBktWaves + 2) * low_bins; k += kThreads) wc[k] = 0;
     __syncthreads();
     {
-        // two rounds of loads in flight: the next round's ids arrive while this round is counted
-        const long round = (long)kThreads * kBktItems;
-        auto fetch = [&](int (&v)[kBktItems], long i0) {
+        const int *first = part_hist + ((long)blockIdx.x - j) * low_bins;
+        const int total = sl.nsl << low_bits;
+        constexpr int kGather = 8;
+        for (int i0 = threadIdx.x; i0 < total; i0 += kThreads * kGather) {
+            int c[kGather];
 #pragma unroll
-            for (int it = 0; it < kBktItems; ++it) {
-                const long i = i0 + (long)it * kThreads + threadIdx.x;
-                v[it] = i < e ? kread(keys, i, packed) : -1;
+            for (int q = 0; q < kGather; ++q) {
+                const int i = i0 + q * kThreads;
+                c[q] = i < total ? first[i] : 0;
             }
-        };
-        auto count = [&](const int (&v)[kBktItems], long i0) {
 #pragma unroll
-            for (int it = 0; it < kBktItems; ++it) {
-                const long i = i0 + (long)it * kThreads + threadIdx.x;
-                const int d = v[it] - u_lo;
-                if (i < e && (unsigned)d < (unsigned)low_bins) {
-                    atomicAdd(&tot[d], 1);
-                    if (i < my_s) atomicAdd(&off[d], 1);
-                }
+            for (int q = 0; q < kGather; ++q) {
+                const int i = i0 + q * kThreads;
+                if (c[q] == 0) continue;
+                const int d = i & (low_bins - 1), k = i >> low_bits;
+                atomicAdd(&tot[d], c[q]);
+                if (k < j) atomicAdd(&off[d], c[q]);
             }
-        };
-        int va[kBktItems], vb[kBktItems];
-        long i0 = s;
-        fetch(va, i0);
-        for (;;) {
-            if (i0 + round >= e) {
-                count(va, i0);
-                break;
-            }
-            fetch(vb, i0 + round);
-            count(va, i0);
-            i0 += round;
-            if (i0 + round >= e) {
-                count(vb, i0);
-                break;
-            }
-            fetch(va, i0 + round);
-            count(vb, i0);
-            i0 += round;
         }
     }
     __syncthreads();
@@ -732,22 +803,14 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
     for (long c0 = my_s; c0 < my_e; c0 += kBktChunk) {
         int key[kBktItems], row[kBktItems], lrank[kBktItems];
         volatile int *mywc = wc + w * low_bins;
-        const long wbase = c0 + (long)w * (64 * kBktItems);
+        if (c0 == my_s) {
 #pragma unroll
-        for (int it = 0; it < kBktItems; ++it) {
-            const long i = wbase + (long)it * 64 + lane;
-            int v = -1;
-            row[it] = (int)i;
-            if (i < my_e) {
-                if (packed) {
-                    const int2 kr = reinterpret_cast<const int2 *>(pairs1)[i];
-                    v = kr.x;
-                    row[it] = kr.y;
-                } else {
-                    v = inv[i];
-                }
+            for (int it = 0; it < kBktItems; ++it) {
+                key[it] = key0[it];
+                row[it] = row0[it];
             }
-            key[it] = (i < my_e && (unsigned)(v - u_lo) < (unsigned)low_bins) ? v : -1;
+        } else {
+            load_round(c0, key, row);
         }
 #pragma unroll
         for (int it = 0; it < kBktItems; ++it) {
@@ -924,7 +987,17 @@ int64_t txs_plan_workspace_len(int64_t num_total, int64_t num_unq) {
     // (id, row) pairs after the bucket scatter, the digit-major histogram, tile flags, bucket
     // boundaries, the scan workspace
     const int64_t hist = bins * (tiles > 0 ? tiles : 1) + 1;
-    const int64_t bucket = 2 * num_total + hist + tiles + bins + 1 + scan_tiles(hist + 1) + 17;
+    // per-slice voxel counts of the bucket kernels: (slices + buckets) * voxels per bucket, for
+    // the digit split txs_plan_build uses
+    const int ubits = radix_bits(num_unq > 1 ? num_unq : 1);
+    int low_bits = ubits <= kBucketLowBitsMax ? 0 : ubits - kBucketHighBits;
+    if (low_bits > kBucketLowBitsMax) low_bits = kBucketLowBitsMax;
+    int64_t counts = 0;
+    if (low_bits > 0 && ubits <= kBucketBitsMax) {
+        const int64_t groups = num_total / kBktSlice + ((int64_t)1 << (ubits - low_bits));
+        counts = 4 + 4 * groups + groups * ((int64_t)1 << low_bits);
+    }
+    const int64_t bucket = 2 * num_total + hist + tiles + bins + 1 + scan_tiles(hist + 1) + 17 + counts;
     return general > bucket ? general : bucket;
 }
 
@@ -982,6 +1055,11 @@ int txs_plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, i
     int *tile_flags = hist + used + 1;
     int *bucket_start = tile_flags + n_tiles;
     int *scan_ws = bucket_start + high_bins + 1;
+    // an upper bound of the (bucket, slice) pairs; workgroups beyond the last pair return at once
+    const long groups = n / kBktSlice + high_bins;
+    int *wg_pick = reinterpret_cast<int *>(  // 16-byte records
+        ((uintptr_t)(scan_ws + scan_tiles(used + 1) + 17) + 15u) & ~(uintptr_t)15u);
+    int *part_hist = wg_pick + 4 * groups;
     static bool lds_allowed = false;
     if (!lds_allowed) {
         for (const void *k : {reinterpret_cast<const void *>(bucket_scatter_kernel<4>),
@@ -1020,11 +1098,12 @@ int txs_plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, i
         nullptr, reinterpret_cast<int2 *>(pairs1));
     const int low_bins = 1 << low_bits;
     const size_t lds = (size_t)(kBktWaves + 2) * low_bins * sizeof(int);
-    // an upper bound of the (bucket, slice) pairs; workgroups beyond the last pair return at once
-    const long groups = n / kBktSlice + high_bins;
+    bucket_count_kernel<<<dim3((unsigned)groups), dim3(kThreads), (size_t)low_bins * sizeof(int), st>>>(
+        unq_inv, pairs1, n, U, low_bits, high_bins, bucket_start, stats, reinterpret_cast<int4 *>(wg_pick), part_hist);
     bucket_plan_kernel<<<dim3((unsigned)groups), dim3(kThreads), lds, st>>>(
         unq_inv, pairs1, n, U, low_bits, high_bins, bucket_start, heavy_threshold,
-        (const long long *)unq_cnts, perm, seg, preSum, slot_of, heavy_ids, stats);
+        (const long long *)unq_cnts, perm, seg, preSum, slot_of, heavy_ids, stats,
+        reinterpret_cast<const int4 *>(wg_pick), part_hist);
     return status_of(hipGetLastError());
 }
 
