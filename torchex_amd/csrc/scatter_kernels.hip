@@ -90,7 +90,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     constexpr bool kMax = OP == TXS_MAX || OP == TXS_MAX_REFTIE;
     // (the fp16 running max keeps packed halves and has registers to spare for a deeper batch)
     constexpr int kBatch = sizeof(raw) == 2 ? ((kMax && std::is_same<TR, F16>::value) ? kBatchHalfMax : kBatchHalf) : ::kBatch;
-    constexpr bool kRef = OP == TXS_MAX_REFTIE;  // idx[] then holds ref_key, not a row
+    constexpr bool kRef = OP == TXS_MAX_REFTIE;  // idx[] then holds the winner's staged position, not its row
     extern __shared__ int lds[];
     const int G = kThreads >> lpr_log2;
     const int T = G * CHUNK;
@@ -187,6 +187,11 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
         idx[k] = -1;
     }
 
+    // What competes in the low word of a heavy voxel's packed key (smaller wins): the row, or in
+    // reference-tie mode the reference's tie key of the winner's offset inside its voxel.
+    auto low_word = [&](int id) -> unsigned {
+        return kRef ? (unsigned)ref_key(rel0 + (id - run_l0), ref_log2) : (unsigned)id;
+    };
     // Emit the finished run [run_l0, run_end) of voxel `cur`.
     auto flush = [&](int run_end) {
         const int u = cur & kIdMask;
@@ -224,7 +229,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                 for (int k = 0; k < VEC; ++k) {
                     r.v[k] = idx[k] >= 0 ? TR::from_m(acc[k]) : TR::lowest();
                     ai.v[k] = idx[k];
-                    if (kRef && idx[k] >= 0) ai.v[k] = row_at(run_l0 + ref_rel(idx[k], ref_log2) - rel0);
+                    if (kRef && idx[k] >= 0) ai.v[k] = row_at(idx[k]);
                 }
                 st_stream<int, VEC>(arg + o, ai);
             }
@@ -238,7 +243,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
             for (int k = 0; k < VEC; ++k) {
                 if constexpr (kMax) {
                     sv[k] = idx[k] >= 0 ? (((unsigned long long)ordered_bits((float)acc[k]) << 32) |
-                                           (unsigned long long)(0xffffffffu - (unsigned)idx[k]))
+                                           (unsigned long long)(0xffffffffu - low_word(idx[k])))
                                         : 0ull;
                 } else {
                     sv[k] = (double)acc[k];
@@ -257,7 +262,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                     if constexpr (kMax) {
                         if (idx[k] >= 0)
                             atomicMax(scratch + o, ((unsigned long long)ordered_bits((float)acc[k]) << 32) |
-                                                       (unsigned long long)(0xffffffffu - (unsigned)idx[k]));
+                                                       (unsigned long long)(0xffffffffu - low_word(idx[k])));
                     } else {
                         unsafeAtomicAdd(reinterpret_cast<float *>(scratch) + o, acc[k]);
                     }
@@ -283,7 +288,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
                 idx[k] = -1;
             }
         }
-        const int tag = kRef ? ref_key(rel0 + (l - run_l0), ref_log2) : row;
+        const int tag = kRef ? l : row;
         if constexpr (!kMax && !kGate && TXS_F16_FMA_MIX && std::is_same<TR, F16>::value && VEC % 2 == 0) {
             unsigned w[VEC / 2 > 0 ? VEC / 2 : 1];
             __builtin_memcpy(w, &v, sizeof(unsigned) * (VEC / 2));
@@ -294,14 +299,33 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
             }
             return;
         }
+        if constexpr (kRef) {
+            // Reference-tie mode also takes an equal value whose tie key is smaller.  Equal
+            // values are rare, so the keys (of this row's offset in its voxel and of the
+            // current winner's) are only worked out where a lane meets one.
+            bool tie = false;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) tie |= TR::to_m(v.v[k]) == acc[k];
+            if (kGate) tie &= valid;
+            if (__builtin_expect(tie, 0)) {
+                const unsigned kn = (unsigned)ref_key(rel0 + (l - run_l0), ref_log2);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    if (!(TR::to_m(v.v[k]) == acc[k])) continue;
+                    const unsigned ko = idx[k] < 0 ? 0xffffffffu : (unsigned)ref_key(rel0 + (idx[k] - run_l0), ref_log2);
+                    if (kn < ko) {  // the value's bits follow the winner (a zero's sign)
+                        idx[k] = tag;
+                        acc[k] = TR::to_m(v.v[k]);
+                    }
+                }
+            }
+        }
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
             if constexpr (kMax) {
                 const AccT x = TR::to_m(v.v[k]);
-                // strict '>': the first row wins ties, NaN never wins.  Reference-tie
-                // mode also takes an equal value whose key is smaller.
+                // strict '>': the first row wins ties, NaN never wins
                 bool take = x > acc[k];
-                if (kRef) take |= (x == acc[k]) && ((unsigned)tag < (unsigned)idx[k]);
                 if (kGate) take &= valid;
                 acc[k] = take ? x : acc[k];
                 idx[k] = take ? tag : idx[k];
