@@ -261,6 +261,19 @@ int txs_counts_from_presum(const int32_t *preSum, int64_t num_unq, int64_t *unq_
 int txs_ingroup_inds(const int32_t *seg, const int32_t *perm, const int32_t *preSum,
                      int64_t num_total, int64_t num_unq, int64_t *out, void *stream);
 
+/* The whole of ingroup_inds (operator_py/ingroup_inds_op.py:10-27) in one call: the index
+ * preparation of the group ids (order and offsets only) and the ranks, queued together; for
+ * up to 2^22 groups the kernels that place the rows write the ranks themselves and leave
+ * perm / seg unwritten.  num_groups: an upper bound of the ids (num_total serves for the
+ * inverse of a unique).  plan_ws, perm, seg, preSum, stats as for txs_plan_build (stats
+ * zero-filled).  On return stats[OUT_OF_RANGE] tells of an id outside [0, num_groups) and
+ * stats[NEED_GENERAL] of a bucket too crowded for the bucket kernels: in both cases `out` is
+ * not valid and the caller ranks again (with the true bound, or through
+ * txs_plan_build_general followed by txs_ingroup_inds). */
+int txs_group_ranks(const int32_t *group_ids, int64_t num_total, int64_t num_groups,
+                    int32_t *plan_ws, int32_t *perm, int32_t *seg, int32_t *preSum, int64_t *out,
+                    int32_t *stats, void *stream);
+
 /* Points inside (enlarged) rotated boxes.  Replaces dynamic_point_pool_launcher
  * (torchex/src/dynamic_point_pool/dynamic_point_pool.cpp:20-32, kernels
  * dynamic_point_pool_kernel.cu:73-170,280-310): for every (box, point) pair with

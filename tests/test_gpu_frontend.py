@@ -200,6 +200,22 @@ def test_ingroup_inds():
     assert np.array_equal(out.cpu().numpy().reshape(-1), orc.ingroup_inds(two_d.reshape(-1).numpy()))
     with pytest.raises(RuntimeError, match="non-negative"):
         T.ingroup_inds(torch.tensor([3, -1, 2], device=DEV))
+    # few groups over many elements (cluster or batch ids): all ids share one bucket of the first
+    # attempt, which guesses the number of elements as their bound; the second attempt, with the
+    # true bound, must rank them (and quickly: the time is bounded loosely here)
+    import time
+    many = torch.randint(0, 1000, (1_000_000,), generator=g)
+    want = orc.ingroup_inds(many.numpy())
+    md = many.to(DEV)
+    assert np.array_equal(T.ingroup_inds(md).cpu().numpy(), want)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    T.ingroup_inds(md)
+    torch.cuda.synchronize()
+    assert time.perf_counter() - t0 < 0.01, "few groups over many elements must not take the slow route"
+    # ... and few groups with huge ids: one crowded bucket also under the true bound
+    far = many * 1_000_000 + 7
+    assert np.array_equal(T.ingroup_inds(far.to(DEV)).cpu().numpy(), want)
 
 
 # ---------------------------------------------------------- dynamic point pool --

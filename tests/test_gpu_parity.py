@@ -839,6 +839,28 @@ def test_mostly_empty_voxel_grid():
     assert ids[0].item() == 123_456 and bool((cnts[ids[1:].long()] == 0).all())
 
 
+def test_long_runs_of_empty_voxels_through_the_general_sequence():
+    """CSR offsets from sorted ids when thousands of consecutive voxels are empty: the general
+    sequence (here forced by one voxel that holds most of the rows) fills such runs block by
+    block.  Offsets, order and the operators against the oracle; first and last voxel empty or
+    not, run lengths around the 256-id block size."""
+    import time
+    g = torch.Generator().manual_seed(91)
+    U, C = 3_000_000, 4
+    used = torch.tensor([0, 1, 255, 256, 257, 511, 512, 513, 1000, 70_000, 70_255, 70_256, 70_767, 70_768,
+                         2_000_000, 2_999_743, 2_999_744, 2_999_999])
+    for name, drop in (("ends used", []), ("first and last empty", [0, U - 1])):
+        ids = torch.tensor([u for u in used.tolist() if u not in drop])
+        crowd = 300_000                                   # one voxel above the bucket kernels' limit
+        inv = torch.cat([ids.repeat(3), torch.full((crowd,), 1000)])
+        inv = inv[torch.randperm(inv.numel(), generator=g)]
+        feats = torch.randint(-4, 5, (inv.numel(), C), generator=g).float()
+        t0 = time.perf_counter()
+        data = run_case(f"empty runs, {name}", feats, inv, torch.bincount(inv, minlength=U))
+        assert data.max_cnt == crowd + 3 and data.num_special == U - ids.numel() + 1
+        assert time.perf_counter() - t0 < 60
+
+
 def test_reference_style_module_calls_reuse_their_plan():
     """scatter_ext.sum / max take only CSR offsets (the reference's signatures).  The
     plan behind a preSum tensor is kept between calls; it is rebuilt when the tensor is

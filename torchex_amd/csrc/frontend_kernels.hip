@@ -182,6 +182,20 @@ __global__ void ingroup_inds_kernel(const int *__restrict__ seg, const int *__re
     if ((unsigned)u < (unsigned)U && (unsigned)row < (unsigned)n) out[row] = (long long)(j - preSum[u]);
 }
 
+// the same from a plan whose order flag is still on the device: stats[UNSORTED] says whether
+// perm was written (rows already in order leave it unwritten: position == row); a plan that
+// was not completed (ids out of range, or handed to the general sequence) is left alone
+__global__ void ingroup_inds_auto_kernel(const int *__restrict__ seg, const int *__restrict__ perm,
+                                         const int *__restrict__ preSum, const int *__restrict__ stats,
+                                         long n, int U, long long *__restrict__ out) {
+    long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    if (stats[TXS_STAT_OUT_OF_RANGE] != 0 || stats[TXS_STAT_NEED_GENERAL] != 0) return;
+    const int u = seg[j] & kIdMask;
+    const int row = stats[TXS_STAT_UNSORTED] != 0 ? perm[j] : (int)j;
+    if ((unsigned)u < (unsigned)U && (unsigned)row < (unsigned)n) out[row] = (long long)(j - preSum[u]);
+}
+
 // ------------------------------------------------------ dynamic point pool --
 // Points inside (enlarged) rotated boxes, with 13 box-relative numbers per hit
 // (torchex/src/dynamic_point_pool/dynamic_point_pool_kernel.cu:22-170,280-310).
@@ -534,6 +548,22 @@ int txs_unique_runs(const int32_t *sorted_keys, const int32_t *perm, int64_t num
     if (exclusive_scan(flags, n, flags, n, scan_ws, st) != hipSuccess) return TXS_ERR_LAUNCH;
     unique_finish_kernel<<<dim3(blocks_for(n)), dim3(kThreads), 0, st>>>(sorted_keys, perm, flags, n, seg,
                                                                        unq_inv, unq_keys, preSum, stats);
+    return status_of(hipGetLastError());
+}
+
+int txs_group_ranks(const int32_t *group_ids, int64_t num_total, int64_t num_groups, int32_t *plan_ws,
+                    int32_t *perm, int32_t *seg, int32_t *preSum, int64_t *out, int32_t *stats, void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_groups) || !stats) return TXS_ERR_INVALID_ARG;
+    if (num_total == 0) return TXS_OK;
+    if (!group_ids || !plan_ws || !perm || !seg || !preSum || !out || num_groups <= 0) return TXS_ERR_INVALID_ARG;
+    const int32_t heavy = txs_default_heavy_threshold();
+    // the bucket kernels rank while they place; any other route leaves a plan to rank from
+    const bool fused = txs_detail::plan_writes_ranks(num_total, num_groups);
+    const int rc = txs_detail::plan_build(group_ids, num_total, num_groups, heavy, nullptr, plan_ws, perm, seg, preSum,
+                                          nullptr, nullptr, stats, fused ? (long long *)out : nullptr, stream);
+    if (rc != TXS_OK || fused) return rc;
+    ingroup_inds_auto_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+        seg, perm, preSum, stats, num_total, (int)num_groups, (long long *)out);
     return status_of(hipGetLastError());
 }
 

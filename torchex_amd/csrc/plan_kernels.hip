@@ -45,8 +45,11 @@ __global__ void copy_if_sorted_kernel(const int *__restrict__ inv, long n,
 }
 
 // CSR offsets from sorted keys: preSum[u] = first position whose key is >= u.
-// Thread j owns the boundary in front of position j and fills the offsets of
-// every id in (key[j-1], key[j]] (more than one only across empty voxels).
+// Thread j owns the boundary in front of position j, i.e. the ids in (key[j-1], key[j]]
+// (more than one only across empty voxels).  A long run of empty voxels is not walked by
+// its one owner: the aligned blocks of kGapBlock ids that lie wholly inside a gap are left to
+// presum_gap_blocks_kernel, and the owner fills only the two ragged ends.
+constexpr int kGapBlock = 256;
 __global__ void presum_from_sorted_kernel(const int *__restrict__ keys, long n, int U,
                                           int *__restrict__ preSum) {
     long j = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -54,8 +57,39 @@ __global__ void presum_from_sorted_kernel(const int *__restrict__ keys, long n, 
     long lo = (j == 0) ? -1 : (long)(keys[j - 1] & kIdMask);
     long hi = (j == n) ? (long)U : (long)(keys[j] & kIdMask);
     if (hi > U) hi = U;
-    for (long u = lo + 1; u <= hi; ++u)
-        if (u >= 0) preSum[u] = (int)j;
+    // whole blocks [b0, b1) of ids inside (lo, hi]
+    const long b0 = (lo + 1 + kGapBlock - 1) / kGapBlock * kGapBlock;
+    const long b1 = (hi + 1) / kGapBlock * kGapBlock;
+    if (b1 > b0) {
+        for (long u = lo + 1; u < b0; ++u) preSum[u] = (int)j;
+        for (long u = b1; u <= hi; ++u) preSum[u] = (int)j;
+    } else {
+        for (long u = lo + 1; u <= hi; ++u) preSum[u] = (int)j;
+    }
+}
+
+// One workgroup per aligned block of kGapBlock ids: if no key falls inside the block (and
+// none equals its last id's successor boundary), every id of it has the same offset, the
+// first position whose key is at or above the block.
+__global__ __launch_bounds__(kGapBlock) void presum_gap_blocks_kernel(const int *__restrict__ keys, long n, int U,
+                                                                      int *__restrict__ preSum) {
+    __shared__ long s_pos;
+    const long bs = (long)blockIdx.x * kGapBlock, be = bs + kGapBlock;  // ids [bs, be)
+    if (be - 1 > (long)U) return;                                       // not wholly inside [0, U]
+    if (threadIdx.x == 0) {
+        long a = 0, b = n;  // first position whose key is >= bs
+        while (a < b) {
+            const long m = (a + b) >> 1;
+            if ((long)(keys[m] & kIdMask) < bs) a = m + 1; else b = m;
+        }
+        // the block lies wholly inside one gap iff the key at that position (or the end of
+        // the ids, U) is at or beyond the block's last id
+        const long next = a < n ? (long)(keys[a] & kIdMask) : (long)U;
+        s_pos = next >= be - 1 ? a : -1;
+    }
+    __syncthreads();
+    const long pos = s_pos;
+    if (pos >= 0) preSum[bs + threadIdx.x] = (int)pos;
 }
 
 // ------------------------------------------------------------ exclusive scan --
@@ -638,7 +672,12 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
     int low_bits, int high_bins, const int *__restrict__ bucket_start, int heavy_threshold,
     const long long *__restrict__ unq_cnts, int *__restrict__ perm, int *__restrict__ seg,
     int *__restrict__ preSum, int *__restrict__ slot_of, int *__restrict__ heavy_ids,
-    int *__restrict__ stats, const int4 *__restrict__ wg_pick, const int *__restrict__ part_hist) {
+    int *__restrict__ stats, const int4 *__restrict__ wg_pick, const int *__restrict__ part_hist,
+    long long *__restrict__ ranks) {
+    // ranks != NULL: the caller wants the rank of every row inside its voxel and nothing else
+    // (ingroup_inds): off[] then counts from the voxel's first row instead of the bucket's,
+    // and the placement writes ranks[row] in place of the permutation and the ids
+    const bool rank_mode = ranks != nullptr;
     extern __shared__ int wc[];  // [kBktWaves][low_bins], tot[low_bins], off[low_bins]
     __shared__ int s_red[kBktWaves], s_bad[kBktWaves];
     const int low_bins = 1 << low_bits;
@@ -734,7 +773,7 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
         const int c = tot[d];
         const int excl = run;
         run += c;
-        off[d] += excl;
+        if (!rank_mode) off[d] += excl;
         if (j == 0 && u_lo + d < u_hi) {
             preSum[u_lo + d] = (int)s + excl;
             if (u_lo + d == U - 1) preSum[U] = (int)n;
@@ -851,7 +890,9 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
             const int dg = key[it] - u_lo;
             atomicAdd(&off[dg], 1);       // the next round starts behind this round's rows
             wc[w * low_bins + dg] = 0;    // (every row of the group stores the same zero)
-            if (dst[it] >= s && dst[it] < e) {
+            if (rank_mode) {
+                if ((unsigned)row[it] < (unsigned)n) ranks[row[it]] = (long long)(dst[it] - s);
+            } else if (dst[it] >= s && dst[it] < e) {
                 const int c = tot[dg];
                 seg[dst[it]] = key[it] | (c > heavy_threshold ? kSpecialBit : 0);
                 if (unsorted) perm[dst[it]] = row[it];
@@ -942,6 +983,10 @@ int txs_plan_presum(const int32_t *sorted_keys, int64_t num_total, int64_t num_u
     if (num_total > 0 && !sorted_keys) return TXS_ERR_INVALID_ARG;
     presum_from_sorted_kernel<<<dim3(blocks_for(num_total + 1)), dim3(kThreads), 0,
                                 (hipStream_t)stream>>>(sorted_keys, num_total, (int)num_unq, preSum);
+    // long runs of empty voxels, one workgroup per 256 ids (only where there can be any)
+    if (num_unq + 1 >= kGapBlock)
+        presum_gap_blocks_kernel<<<dim3((unsigned)((num_unq + 1) / kGapBlock)), dim3(kGapBlock), 0,
+                                   (hipStream_t)stream>>>(sorted_keys, num_total, (int)num_unq, preSum);
     return status_of(hipGetLastError());
 }
 
@@ -1025,6 +1070,24 @@ int txs_plan_build_general(const int32_t *unq_inv, int64_t num_total, int64_t nu
 int txs_plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, int32_t heavy_threshold,
                    const int64_t *unq_cnts, int32_t *plan_ws, int32_t *perm, int32_t *seg, int32_t *preSum,
                    int32_t *slot_of, int32_t *heavy_ids, int32_t *stats, void *stream) {
+    return txs_detail::plan_build(unq_inv, num_total, num_unq, heavy_threshold, unq_cnts, plan_ws, perm, seg, preSum,
+                                  slot_of, heavy_ids, stats, nullptr, stream);
+}
+
+}  // extern "C"
+
+// txs_plan_build, or with `ranks` the in-voxel rank of every row and no special-voxel table.
+// Ranks are written by the bucket kernels only: txs_detail::plan_writes_ranks tells a caller
+// whether they apply to the extents (otherwise it ranks from the plan this call leaves).
+bool txs_detail::plan_writes_ranks(long num_total, long num_unq) {
+    const int bits = radix_bits(num_unq > 1 ? num_unq : 1);
+    return num_total > 0 && num_unq > 0 && bits <= kBucketBitsMax && bits > kBucketLowBitsMax;
+}
+
+int txs_detail::plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, int32_t heavy_threshold,
+                           const int64_t *unq_cnts, int32_t *plan_ws, int32_t *perm, int32_t *seg,
+                           int32_t *preSum, int32_t *slot_of, int32_t *heavy_ids, int32_t *stats,
+                           long long *ranks, void *stream) {
     if (!fits_i32(num_total) || !fits_i32(num_unq) || !stats || !preSum || heavy_threshold < kChunk)
         return TXS_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
@@ -1103,8 +1166,6 @@ int txs_plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, i
     bucket_plan_kernel<<<dim3((unsigned)groups), dim3(kThreads), lds, st>>>(
         unq_inv, pairs1, n, U, low_bits, high_bins, bucket_start, heavy_threshold,
         (const long long *)unq_cnts, perm, seg, preSum, slot_of, heavy_ids, stats,
-        reinterpret_cast<const int4 *>(wg_pick), part_hist);
+        reinterpret_cast<const int4 *>(wg_pick), part_hist, ranks);
     return status_of(hipGetLastError());
 }
-
-}  // extern "C"

@@ -306,35 +306,39 @@ Tensor group_ranks(const Tensor &ids_in) {
     Tensor out = at::empty({N}, ids.options().dtype(at::kLong));
     if (N == 0) return out;
     void *st = cur_stream(ids);
-    auto attempt = [&](int64_t U) -> bool {
+    // `exact`: U is the true bound of the ids (largest id + 1), not the guess `number of rows`
+    auto attempt = [&](int64_t U, bool exact) -> bool {
         Tensor stats = at::zeros({TXS_STATS_LEN}, ids.options());
         Tensor seg = empty_i32(N, ids), perm = empty_i32(N, ids);
         Tensor preSum = empty_i32(U + 1, ids);
         Tensor ws = empty_i32(txs_plan_workspace_len(N, U), ids);
         const int32_t heavy = txs_default_heavy_threshold();
-        // order and offsets only: no special-voxel table
-        check_status(txs_plan_build(i32p(ids), N, U, heavy, nullptr, i32w(ws), i32w(perm), i32w(seg), i32w(preSum),
-                                    nullptr, nullptr, i32w(stats), st),
-                     "plan_build");
+        // order and offsets only (no special-voxel table) and the ranks, queued together
+        check_status(txs_group_ranks(i32p(ids), N, U, i32w(ws), i32w(perm), i32w(seg), i32w(preSum),
+                                     out.data_ptr<int64_t>(), i32w(stats), st),
+                     "group_ranks");
         std::vector<int64_t> hs = read_stats(stats);
         if (hs[TXS_STAT_OUT_OF_RANGE]) return false;
         if (hs[TXS_STAT_NEED_GENERAL]) {
+            // one bucket holds most of the rows.  Under the guessed bound that usually means few
+            // groups with small ids: the true bound gives narrower buckets, often none to sort by
+            if (!exact) return false;
             stats.zero_();
             check_status(txs_plan_build_general(i32p(ids), N, U, heavy, nullptr, i32w(ws), i32w(perm), i32w(seg),
                                                 i32w(preSum), nullptr, nullptr, i32w(stats), st),
                          "plan_build_general");
             hs = read_stats(stats);
+            // ids already in order leave perm unwritten: position == row
+            check_status(txs_ingroup_inds(i32p(seg), hs[TXS_STAT_UNSORTED] ? i32p(perm) : nullptr, i32p(preSum), N, U,
+                                          out.data_ptr<int64_t>(), st),
+                         "ingroup_inds");
         }
-        // ids already in order leave perm unwritten: position == row
-        check_status(txs_ingroup_inds(i32p(seg), hs[TXS_STAT_UNSORTED] ? i32p(perm) : nullptr, i32p(preSum), N, U,
-                                      out.data_ptr<int64_t>(), st),
-                     "ingroup_inds");
         return true;
     };
-    if (!attempt(N)) {
+    if (!attempt(N, false)) {
         const int64_t lo = ids.min().item<int64_t>(), hi = ids.max().item<int64_t>();
         TORCH_CHECK(lo >= 0, "group_inds must be non-negative");
-        TORCH_CHECK(attempt(hi + 1), "group_inds could not be ranked");
+        TORCH_CHECK(attempt(hi + 1, true), "group_inds could not be ranked");
     }
     return out;
 }

@@ -261,6 +261,14 @@ long scan_tiles(long n_out);
 hipError_t exclusive_scan(const int *in, long n_in, int *out, long n_out, int *ws, hipStream_t st);
 
 
+// txs_plan_build with one more output (plan_kernels.hip): ranks != NULL asks for the rank of
+// every row inside its voxel instead of the permutation and the per-position ids; only the
+// bucket kernels write it, which plan_writes_ranks() predicts from the extents.
+int plan_build(const int32_t *unq_inv, int64_t num_total, int64_t num_unq, int32_t heavy_threshold,
+               const int64_t *unq_cnts, int32_t *plan_ws, int32_t *perm, int32_t *seg, int32_t *preSum,
+               int32_t *slot_of, int32_t *heavy_ids, int32_t *stats, long long *ranks, void *stream);
+bool plan_writes_ranks(long num_total, long num_unq);
+
 // Row-order "table mode" for inputs with few voxels (table_kernels.hip): whether it
 // applies to a call and with which launch geometry.
 struct TablePlan {
