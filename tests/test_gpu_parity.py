@@ -625,6 +625,31 @@ def test_reference_tie_rule_mode(sizes):
     assert bits_equal(x.grad.cpu().numpy(), orc.max_backward(gup.numpy(), want_arg_s, N))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_reference_tie_rule_special_values_and_half_precision(dtype):
+    """Grouped rows (the reference's input, so its tie rule is in force) full of equal values,
+    signed zeros, infinities and NaN, in every dtype, through registers and through the heavy-voxel
+    table: arg and the value's bits against the lane-exact emulation of the reference kernel."""
+    g = torch.Generator().manual_seed(55)
+    sizes = [1, 2, 17, 33, 64, 65, 100, 300, 1500, 40, 3, 700]
+    U, C = len(sizes), 10
+    inv = torch.repeat_interleave(torch.arange(U), torch.tensor(sizes))
+    N = inv.numel()
+    f = torch.randint(-3, 4, (N, C), generator=g).float()          # few distinct values: ties everywhere
+    f[torch.rand((N, C), generator=g) < 0.10] = -0.0
+    f[torch.rand((N, C), generator=g) < 0.05] = float("nan")
+    f[torch.rand((N, C), generator=g) < 0.03] = float("inf")
+    f[torch.rand((N, C), generator=g) < 0.05] = float("-inf")
+    f[inv == 9] = float("-inf")                                     # a voxel without a finite value
+    f[inv == 10] = float("nan")
+    cnts = torch.tensor(sizes)
+    for thr in (None, 1 << 20):
+        with np.errstate(invalid="ignore"):   # inf - inf in the checks of the sums
+            data = run_case(f"reference ties, special values, threshold {thr}", f, inv, cnts, dtype=dtype,
+                            heavy_threshold=thr)
+        assert data.max_tie_rule == "reference"
+
+
 def test_reference_tie_rule_mode_matches_default_without_ties():
     T = tx()
     w = workloads.lidar_sweep(N=200_000, C=32, seed=12)
