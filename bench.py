@@ -172,8 +172,9 @@ def frontend_timings(T, workloads, dev, N):
     keys_cpu, key_bound = workloads._lidar_keys(N, torch.Generator().manual_seed(2))
     keys = keys_cpu.to(dev)
 
-    def wall_ms(fn, iters=5):
-        fn()
+    def wall_ms(fn, iters=20):
+        for _ in range(3):
+            fn()
         torch.cuda.synchronize()
         t = time.perf_counter()
         for _ in range(iters):

@@ -275,6 +275,7 @@ constexpr int kDppBoxesPerWg = 8;
 __global__ __launch_bounds__(kThreads) void dpp_count_kernel(const float *__restrict__ pts, int P,
                                                              const DppBox *__restrict__ boxes, int B,
                                                              int n_tiles, int *__restrict__ counts,
+                                                             unsigned short *__restrict__ flags16,
                                                              const int *__restrict__ pts_batch,
                                                              const int *__restrict__ rois_batch) {
     __shared__ int cnt[kDppBoxesPerWg];
@@ -290,16 +291,21 @@ __global__ __launch_bounds__(kThreads) void dpp_count_kernel(const float *__rest
         z = pts[(size_t)p * 3 + 2];
         if (pts_batch) sample = pts_batch[p];
     }
+    // the result of every test (2 bits per box of the group) is kept for the second pass,
+    // which so repeats the arithmetic only for the hits it writes
+    unsigned flags = 0u;
     for (int bb = 0; bb < kDppBoxesPerWg && b0 + bb < B; ++bb) {
         const DppBox bx = boxes[b0 + bb];
-        bool hit = false;
+        int flag = 0;
         if (p < P && (!rois_batch || rois_batch[b0 + bb] == sample) && dpp_near(bx, x, y)) {
             float lx, ly;
-            hit = dpp_test(bx, x, y, z, lx, ly) > 0;
+            flag = dpp_test(bx, x, y, z, lx, ly);
         }
-        const int c = __popcll(__ballot(hit));
+        flags |= (unsigned)flag << (2 * bb);
+        const int c = __popcll(__ballot(flag > 0));
         if (c && (threadIdx.x & 63) == 0) atomicAdd(&cnt[bb], c);
     }
+    if (p < P) flags16[(size_t)blockIdx.y * P + p] = (unsigned short)flags;
     __syncthreads();
     if (threadIdx.x < kDppBoxesPerWg && b0 + (int)threadIdx.x < B)
         counts[(size_t)(b0 + threadIdx.x) * n_tiles + blockIdx.x] = cnt[threadIdx.x];
@@ -323,40 +329,26 @@ __global__ __launch_bounds__(kThreads) void dpp_box_base_kernel(const int *__res
     if (threadIdx.x == 0) total_out[0] = min(carry, max_all);
 }
 
-// second pass: same test, rank of the hit inside its box, compact write
+// second pass: rank of every hit inside its box from the first pass's results, compact write
 __global__ __launch_bounds__(kThreads) void dpp_write_kernel(
     const float *__restrict__ pts, int P, const DppBox *__restrict__ boxes, int B, int n_tiles,
     const int *__restrict__ scanned, const int *__restrict__ box_base, int cap, int max_all,
-    long long *__restrict__ out_pts_idx, long long *__restrict__ out_roi_idx,
-    float *__restrict__ out_feats, const int *__restrict__ pts_batch, const int *__restrict__ rois_batch) {
+    const unsigned short *__restrict__ flags16, long long *__restrict__ out_pts_idx,
+    long long *__restrict__ out_roi_idx, float *__restrict__ out_feats) {
 #pragma clang fp contract(off)
     __shared__ int wsum[kDppBoxesPerWg][kThreads / 64];
     const int b0 = blockIdx.y * kDppBoxesPerWg;
     const int p = blockIdx.x * kThreads + threadIdx.x;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    float x = 0.f, y = 0.f, z = 0.f;
-    int sample = 0;
-    if (p < P) {
-        x = pts[(size_t)p * 3];
-        y = pts[(size_t)p * 3 + 1];
-        z = pts[(size_t)p * 3 + 2];
-        if (pts_batch) sample = pts_batch[p];
-    }
-    // phase 1: the test against every box of the group (2 result bits per box) and the
-    // hits of each wave
-    unsigned flags = 0u;
+    // phase 1: the hits of each wave per box of the group
+    const unsigned flags = p < P ? (unsigned)flags16[(size_t)blockIdx.y * P + p] : 0u;
     for (int bb = 0; bb < kDppBoxesPerWg && b0 + bb < B; ++bb) {
-        const DppBox bx = boxes[b0 + bb];
-        int flag = 0;
-        if (p < P && (!rois_batch || rois_batch[b0 + bb] == sample) && dpp_near(bx, x, y)) {
-            float lx, ly;
-            flag = dpp_test(bx, x, y, z, lx, ly);
-        }
-        flags |= (unsigned)flag << (2 * bb);
-        const unsigned long long m = __ballot(flag > 0);
+        const unsigned long long m = __ballot(((flags >> (2 * bb)) & 3u) != 0u);
         if (lane == 0) wsum[bb][w] = __popcll(m);
     }
     __syncthreads();
+    if (flags == 0u) return;  // (no barrier follows)
+    const float x = pts[(size_t)p * 3], y = pts[(size_t)p * 3 + 1], z = pts[(size_t)p * 3 + 2];
     // phase 2: rank of each hit inside its box, compact write (hits are rare)
     for (int bb = 0; bb < kDppBoxesPerWg && b0 + bb < B; ++bb) {
         const int flag = (int)((flags >> (2 * bb)) & 3u);
@@ -580,9 +572,11 @@ int txs_ingroup_inds(const int32_t *seg, const int32_t *perm, const int32_t *pre
 int64_t txs_dpp_workspace_len(int64_t num_pts, int64_t num_boxes) {
     const int64_t tiles = (num_pts + kThreads - 1) / kThreads;
     const int64_t cells = num_boxes * tiles + 1;
-    // box constants, (box, tile) counts, scan workspace, box bases
-    return (int64_t)(sizeof(DppBox) / sizeof(int)) * num_boxes + cells + scan_tiles(cells + 1) + 1 +
-           num_boxes + 16;
+    // box constants, (box, tile) counts, scan workspace, box bases, and the first pass's test
+    // results: 2 bits per (point, box), 16 bits per point and group of 8 boxes
+    const int64_t groups = (num_boxes + kDppBoxesPerWg - 1) / kDppBoxesPerWg;
+    return (int64_t)(sizeof(DppBox) / sizeof(int)) * num_boxes + cells + scan_tiles(cells + 2) + 1 +
+           num_boxes + 16 + (groups * num_pts + 1) / 2;
 }
 
 int txs_dynamic_point_pool(const float *rois, const float *pts, int64_t num_boxes, int64_t num_pts,
@@ -618,17 +612,18 @@ int txs_dynamic_point_pool_mixed(const float *rois, const int32_t *rois_batch, c
     int *counts = workspace + (sizeof(DppBox) / sizeof(int)) * (size_t)B;
     int *scan_ws = counts + cells + 1;
     int *box_base = scan_ws + scan_tiles(cells + 2) + 1;
+    unsigned short *flags16 = reinterpret_cast<unsigned short *>(box_base + B);
     dpp_box_kernel<<<dim3(blocks_for(B)), dim3(kThreads), 0, st>>>(rois, B, extra_wlh[0], extra_wlh[1],
                                                                  extra_wlh[2], boxes);
     const int box_groups = (B + kDppBoxesPerWg - 1) / kDppBoxesPerWg;
     dpp_count_kernel<<<dim3(n_tiles, box_groups), dim3(kThreads), 0, st>>>(pts, P, boxes, B, n_tiles, counts,
-                                                                           pts_batch, rois_batch);
+                                                                           flags16, pts_batch, rois_batch);
     if (exclusive_scan(counts, cells, counts, cells + 1, scan_ws, st) != hipSuccess) return TXS_ERR_LAUNCH;
     dpp_box_base_kernel<<<dim3(1), dim3(kThreads), 0, st>>>(counts, B, n_tiles, max_pts_per_box,
                                                            (int)max_all_pts, box_base, num_out);
     dpp_write_kernel<<<dim3(n_tiles, box_groups), dim3(kThreads), 0, st>>>(
-        pts, P, boxes, B, n_tiles, counts, box_base, max_pts_per_box, (int)max_all_pts,
-        (long long *)out_pts_idx, (long long *)out_roi_idx, out_pts_feats, pts_batch, rois_batch);
+        pts, P, boxes, B, n_tiles, counts, box_base, max_pts_per_box, (int)max_all_pts, flags16,
+        (long long *)out_pts_idx, (long long *)out_roi_idx, out_pts_feats);
     return status_of(hipGetLastError());
 }
 
