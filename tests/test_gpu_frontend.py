@@ -48,12 +48,14 @@ def test_voxelize_matches_torch_floor_division():
     assert np.array_equal(got.numpy(), oc)
 
 
-@pytest.mark.parametrize("case", ["lidar", "sorted", "few_keys", "single", "sparse_ids"])
+@pytest.mark.parametrize("case", ["lidar", "pillars", "sorted", "few_keys", "single", "sparse_ids"])
 def test_from_keys_equals_torch_unique_and_scatter_data(case):
     T = tx()
     g = torch.Generator().manual_seed(7)
-    if case == "lidar":
-        keys, bound = workloads._lidar_keys(300_000, g)
+    if case == "lidar":       # the voxel keys of the LiDAR-like sweep at its full size
+        keys, bound = workloads._lidar_keys(1_000_000, g)
+    elif case == "pillars":   # fewer cells than points
+        keys, bound = workloads._lidar_keys(1_000_000, g, pillars=True)
     elif case == "sorted":
         keys = torch.sort(torch.randint(0, 5000, (50_000,), generator=g)).values
         bound = 5000
