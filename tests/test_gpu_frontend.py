@@ -174,7 +174,8 @@ def test_from_points_end_to_end_and_range_check():
 def test_ingroup_inds():
     T = tx()
     g = torch.Generator().manual_seed(13)
-    for n, ngroups in [(1, 1), (1000, 1), (50_000, 300), (200_000, 150_000)]:
+    # (400k elements in 2048 groups: two buckets of 200k rows, slices of two placement rounds)
+    for n, ngroups in [(1, 1), (1000, 1), (50_000, 300), (200_000, 150_000), (400_000, 2048)]:
         ids = torch.randint(0, ngroups, (n,), generator=g)
         say(f"[case] ingroup_inds n={n} groups={ngroups}")
         out = T.ingroup_inds(ids.to(DEV))
