@@ -96,6 +96,23 @@ def test_argument_validation_needs_no_gpu():
     assert buf.value == b"scatter_fwd_kernel<F16,4,SUM,32>"
     rc = lib.txs_get_presum(vp(0), vp(0), i64(-1), i64(0), vp(0))
     assert rc == 1
+    # the unique-by-occupancy-map and ranking entry points: sizes and null pointers are checked first
+    lib.txs_unique_bitmap_workspace_len.restype = ctypes.c_int64
+    words = (16_875_000 + 31) // 32
+    assert lib.txs_unique_bitmap_workspace_len(i64(16_875_000)) >= 10 * words
+    assert lib.txs_unique_bitmap_workspace_len(i64(0)) == -1
+    assert lib.txs_unique_bitmap_workspace_len(i64((1 << 31) + 1)) == -1
+    assert lib.txs_unique_bitmap_count(vp(0), ci(0), i64(5), i64(0), vp(0), vp(0), vp(0)) == 1
+    assert lib.txs_unique_bitmap_count(vp(0), ci(0), i64(5), i64(100), vp(0), vp(8), vp(0)) == 1   # no keys
+    assert lib.txs_unique_bitmap_assign(vp(0), ci(1), i64(1 << 40), i64(100), vp(0), vp(0), vp(0), vp(0)) == 1
+    assert lib.txs_counts_from_presum(vp(0), i64(3), vp(0), vp(0)) == 1
+    assert lib.txs_counts_from_presum(vp(0), i64(0), vp(0), vp(0)) == 0                             # nothing to do
+    assert lib.txs_group_ranks(vp(0), i64(10), i64(10), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0), vp(0)) == 1
+    lib.txs_plan_workspace_len.restype = ctypes.c_int64
+    assert lib.txs_plan_workspace_len(i64(1_000_000), i64(326_859)) > 2 * 1_000_000
+    lib.txs_dpp_workspace_len.restype = ctypes.c_int64
+    # room for 2 result bits per (point, box): 25 groups of 8 boxes x 200k points x 16 bits
+    assert lib.txs_dpp_workspace_len(i64(200_000), i64(200)) * 4 >= 25 * 200_000 * 2
 
 
 def test_package_surface_matches_reference_exports():
