@@ -1,5 +1,6 @@
 // The callers on either side of the scatter operators: voxel keys from points,
-// the unique / inverse / counts triple (from the same sort the scatter plan uses),
+// the unique / inverse / counts triple (from an occupancy map of the key grid, or from
+// the same sort the scatter plan uses),
 // the rank of an element inside its group, points-in-boxes pooling, and the
 // coordinate hash table.
 //

@@ -1,8 +1,9 @@
 // Index preparation for the voxel scatter kernels (built once per ScatterData and
-// reused by every forward/backward call): sortedness/range check, stable LSD radix
-// sort of (voxel id, row), CSR offsets from run boundaries, table of special
-// voxels, per-position voxel ids.  No histogram atomics on global memory and no
-// inter-block spinning anywhere.
+// reused by every forward/backward call): a two-level bucket sort of (voxel id, row) for up
+// to 2^22 voxels that yields CSR offsets, the table of special voxels and the
+// per-position voxel ids on the way; for anything else a general sequence of
+// sortedness/range check, stable LSD radix sort, CSR offsets from run boundaries and the
+// same tables.  No histogram atomics on global memory and no inter-block spinning anywhere.
 //
 // Reference behaviour being replaced: ScatterData.__init__
 // (torchex/operator_py/scatter_op.py:7-21) and getPreSum
