@@ -15,11 +15,13 @@ durations are measured inside a second pass over the same steps, with a HIP even
 between the four entry-point calls; per-operator times, GB/s and roofline fractions
 derived from them are in ``per_kernel`` / ``per_op``.
 
-``other_configs`` holds the same measurements, GPU only and over fewer steps, for the
-other configurations: the uniform box, the half-precision sweep (fp16, bf16), the Zipf
+``other_configs`` holds the same measurements (``--other-steps`` timed steps each, mean,
+median and minimum per kernel) for the other configurations: the uniform box (with the
+same step on the host cores next to it), the half-precision sweep (fp16, bf16), the Zipf
 contention case, the four-sweep batch and the pillar binning of the sweep (the same
 points in 0.2 m x 0.2 m columns: the heavy-tailed occupancy, two thirds of the points in
-voxels that are split across wavefronts).
+voxels that are split across wavefronts).  ``ms_per_step_graph`` is the step's four
+entry-point calls replayed from a HIP graph (no host work per call).
 
 Prints ONE JSON line on stdout.
 """
@@ -65,7 +67,8 @@ def parse():
     p.add_argument("--no-frontend", action="store_true", help="skip the front-end timings")
     p.add_argument("--no-other-configs", action="store_true",
                    help="measure the selected workload only (profiles of one workload use this)")
-    p.add_argument("--other-steps", type=int, default=12, help="timed steps per entry of other_configs")
+    p.add_argument("--other-steps", type=int, default=50, help="timed steps per entry of other_configs")
+    p.add_argument("--other-warmup", type=int, default=10, help="warm-up steps per entry of other_configs")
     p.add_argument("--sorted-input", action="store_true",
                    help="also time the step on the same points delivered grouped by voxel "
                         "(off by default so that a profile of the default command holds one "
@@ -97,16 +100,17 @@ def event_ms(fn, iters, warm=5):
     return start.elapsed_time(stop) / iters
 
 
-def cpu_baseline(w, g_mean, g_max):
+def cpu_baseline(w, g_mean, g_max, budget_s=12.0):
     """The same step with stock torch CPU ops (scatter_reduce / index_add / gather) on
-    the host cores: a bounded sample of the same workload."""
+    the host cores: a bounded sample of the same workload (about ``budget_s`` seconds of
+    multi-threaded steps, then one step on one thread and one of the C oracle)."""
     from oracle import torch_oracle as tor
     threads = os.cpu_count() or 1
     threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
     torch.set_num_threads(threads)
     tor.step_mean_max(w.feats, w.unq_inv, w.unq_cnts, g_mean, g_max)   # warm-up
     iters, t0 = 0, time.perf_counter()
-    while iters < 3 or (time.perf_counter() - t0 < 12.0 and iters < 40):
+    while iters < 3 or (time.perf_counter() - t0 < budget_s and iters < 40):
         tor.step_mean_max(w.feats, w.unq_inv, w.unq_cnts, g_mean, g_max)
         iters += 1
     dt = (time.perf_counter() - t0) / iters
@@ -162,6 +166,37 @@ def instrumented_steps(scatter_ext, f, g_mean, g_max, plan, bplan, steps, warmup
     mean = {n: sum(v) / len(v) for n, v in per.items()}
     spread = {n: {"median_ms": v[len(v) // 2], "min_ms": v[0]} for n, v in per.items()}
     return mean, spread
+
+
+def graph_step_ms(scatter_ext, f, g_mean, g_max, plan, bplan, steps, warmup):
+    """The step's four entry-point calls recorded once into a HIP graph and replayed: what
+    the step costs when the host's per-call work (argument checks, output allocation,
+    launches) is taken out.  The entry points only launch kernels, so they capture."""
+    def raw_step():
+        scatter_ext.forward(scatter_ext.MEAN, f, *plan)
+        scatter_ext.backward(scatter_ext.MEAN, g_mean, None, *bplan)
+        _, a2 = scatter_ext.forward(scatter_ext.MAX, f, *plan)
+        scatter_ext.backward(scatter_ext.MAX, g_max, a2, *bplan)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        raw_step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        raw_step()
+    for _ in range(max(warmup, 1)):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    del graph
+    return ms
 
 
 def frontend_timings(T, workloads, dev, N):
@@ -309,9 +344,11 @@ def measure(T, scatter_ext, workloads, names, w, dtype, steps, warmup, dev, extr
     bplan = data.backward_args()
     kt, kt_spread = instrumented_steps(scatter_ext, f, g_mean, g_max, plan, bplan, steps, warmup)
     kernel_sum_ms = sum(kt.values())
+    graph_ms = graph_step_ms(scatter_ext, f, g_mean, g_max, plan, bplan, steps, warmup)
     res = {"N": N, "C": C, "U": U, "esz": esz, "data": data, "f": f, "g_mean": g_mean, "g_max": g_max,
            "g_mean_cpu": g_mean_cpu, "g_max_cpu": g_max_cpu, "inv": inv, "cnts": cnts, "plan": plan,
-           "bplan": bplan, "prep_ms": prep_ms, "ms_per_step": ms_per_step, "kernel_sum_ms": kernel_sum_ms}
+           "bplan": bplan, "prep_ms": prep_ms, "ms_per_step": ms_per_step, "kernel_sum_ms": kernel_sum_ms,
+           "ms_per_step_graph": graph_ms}
     if extras:
         # not part of the step: back-to-back launches of scatter_sum's kernels and of the
         # forward under the reference's tie rule (what grouped input gets by default)
@@ -352,10 +389,12 @@ def compact(name, dtype, r):
         "U": r["U"], "max_cnt": r["data"].max_cnt, "num_heavy": r["data"].num_heavy,
         "points_in_heavy_voxels": int(r["cnts"][r["cnts"] > r["data"].heavy_threshold].sum()),
         "ms_per_step": r["ms_per_step"], "kernel_sum_ms": r["kernel_sum_ms"],
+        "ms_per_step_graph": r["ms_per_step_graph"],
         "points_per_s": 2 * r["N"] / r["ms_per_step"] * 1e3,
         "step_frac_of_hbm_peak": step_bytes / r["kernel_sum_ms"] / 1e6 / HBM_PEAK_GBPS,
         "per_op_frac": {op: v["frac_of_hbm_peak"] for op, v in r["per_op"].items()},
-        "per_kernel": {k: {"ms": v["ms"], "frac": v["frac"]} for k, v in r["per_kernel"].items()},
+        "per_kernel": {k: {"ms": v["ms"], "frac": v["frac"], "median_ms": v.get("median_ms"),
+                           "min_ms": v.get("min_ms")} for k, v in r["per_kernel"].items()},
         "dominant_kernel": r["per_kernel"][dom]["kernel"], "dominant_frac": r["per_kernel"][dom]["frac"],
         "index_prep_ms": r["prep_ms"],
     }
@@ -374,7 +413,7 @@ def main():
     import __graft_entry__
     __graft_entry__._load_build().ensure_built()
     import torchex_amd as T
-    from torchex_amd import workloads
+    from tests import workloads
     from torchex_amd._native import scatter_ext
 
     dev = torch.device("cuda:0")
@@ -450,6 +489,7 @@ def main():
         "per_op": r["per_op"],
         "per_kernel": per_kernel,
         "kernel_sum_ms": r["kernel_sum_ms"],
+        "ms_per_step_graph": r["ms_per_step_graph"],
         "sorted_input": sorted_input,
         "device_copy_GBps": copy_gbps,
         "index_prep_ms": r["prep_ms"],
@@ -468,8 +508,12 @@ def main():
             if (name, dt) == (a.workload, a.dtype):
                 continue
             wo = w if name == a.workload else make_workload(workloads, name, 1_000_000, 128)
-            ro = measure(T, scatter_ext, workloads, names, wo, dt, a.other_steps, 3, dev)
-            others.append(compact(name, dt, ro))
+            ro = measure(T, scatter_ext, workloads, names, wo, dt, a.other_steps, a.other_warmup, dev)
+            entry = compact(name, dt, ro)
+            if name == "uniform_box" and dt == "f32" and not a.no_cpu_baseline:
+                # the configuration quoted "on the CPU reference path": the same step on the host cores
+                entry["cpu_baseline"] = cpu_baseline(wo, ro["g_mean_cpu"], ro["g_max_cpu"], budget_s=3.0)
+            others.append(entry)
             del ro, wo
             torch.cuda.empty_cache()
         out["other_configs"] = others

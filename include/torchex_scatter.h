@@ -6,8 +6,12 @@
  * (a hipStream_t passed as void*; NULL = the null stream) and an int status.
  * No torch type crosses this line.  The library allocates no device memory:
  * every buffer, workspaces included, is owned by the caller.  Calls are
- * asynchronous on `stream` and re-entrant (no global state), with one exception
- * that says so: txs_scatter_forward_resident, which uses a table inside the library.
+ * asynchronous on `stream` and re-entrant, with one exception that says so:
+ * txs_scatter_forward_resident, which uses a table inside the library.
+ * State the library keeps, all of it per GPU, filled on first use and never changed
+ * afterwards (so it does not make two calls depend on each other): the number of
+ * compute units (sizes the table-mode launch), a flag per kernel that its dynamic-LDS
+ * limit has been raised, and the device address of the resident table.
  *
  * Each entry point names the reference interface it stands in for
  * (paths relative to the TorchEx tree).
@@ -166,8 +170,9 @@ int txs_plan_special(const int32_t *preSum, int64_t num_unq, int32_t heavy_thres
  * bucket sort -- tile histograms of the high digit of the ids; scan; stable scatter by
  * bucket; then workgroups that sort a bucket's low digit in LDS and write the bucket's
  * slice of all outputs -- beyond that it runs the calls named above.
- * stats [TXS_STATS_LEN] needs no initialisation for up to 2^22 voxels and must be
- * zero-filled by the caller beyond (zero-filling always is fine); perm is left unwritten when
+ * stats [TXS_STATS_LEN] needs no initialisation for up to 2^22 voxels (also with no rows or
+ * no voxels at all: the call clears it) and must be zero-filled by the caller beyond
+ * (zero-filling always is fine); perm is left unwritten when
  * stats[UNSORTED] stays 0.  unq_cnts may be NULL.  slot_of and heavy_ids may both be NULL
  * for a caller that wants the order and the offsets only (the ranks of ingroup_inds): no
  * special-voxel table is made then, seg carries plain ids, and of the statistics only

@@ -9,7 +9,7 @@ import torch
 
 from oracle import c_oracle as orc
 from oracle import torch_oracle as tor
-from torchex_amd import workloads
+from tests import workloads
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -129,6 +129,16 @@ def test_from_keys_occupancy_map_and_sort_agree():
         for b in (bound, 2 ** 30) if bad_key < 0 else (bound,):
             with pytest.raises(RuntimeError, match="outside the grid"):
                 T.ScatterData.from_keys(bad.to(DEV), b)
+    # an int64 key whose low 32 bits would pass for a valid one: rejected on both routes
+    # (occupancy map for a grid near the input's size, sort for a much larger bound)
+    for b in (bound, 2 ** 30):
+        bad = keys.clone()
+        bad[77] = 2 ** 32 + 5
+        with pytest.raises(RuntimeError, match="outside the grid"):
+            T.ScatterData.from_keys(bad.to(DEV), b)
+        bad[77] = -(2 ** 32) + 5
+        with pytest.raises(RuntimeError, match="outside the grid"):
+            T.ScatterData.from_keys(bad.to(DEV), b)
     # every cell of a small grid occupied, and a grid of one cell
     full = torch.randperm(4096, generator=g).repeat(3)
     d = T.ScatterData.from_keys(full.to(DEV), 4096)
@@ -429,3 +439,94 @@ def test_grid_hash_class_follows_the_reference_test():
     h = T.GridHash(keys.to(DEV))
     unq, inv = torch.unique(keys, return_inverse=True)
     assert torch.equal(h.probe(keys.to(DEV)).cpu().long(), inv)
+
+
+# ------------------------------- the reference's extension-module names and signatures --
+#
+# The reference's wrappers bind three more modules by name: `import ingroup_indices`
+# (operator_py/ingroup_inds_op.py:4), `import dynamic_point_pool_ext`
+# (operator_py/dynamic_point_pool_op.py:7), `import grid_hash_ext` (operator_py/grid_hash.py:2).
+# Each test below does what the body of the wrapper's forward() does, with
+# caller-allocated outputs where the reference has them, and checks against the oracle.
+
+def test_reference_module_ingroup_indices_forward_in_place():
+    tx()
+    import ingroup_indices
+    g = torch.Generator().manual_seed(31)
+    for n, ngroups in [(1, 1), (70_000, 900), (300_000, 200_000)]:
+        group_inds = torch.randint(0, ngroups, (n,), generator=g).to(DEV)
+        say(f"[case] ingroup_indices.forward n={n} groups={ngroups}")
+        out_inds = torch.zeros_like(group_inds) - 1                  # ingroup_inds_op.py:15
+        assert ingroup_indices.forward(group_inds, out_inds) is None  # :17
+        assert out_inds.dtype == torch.int64
+        assert np.array_equal(out_inds.cpu().numpy(), orc.ingroup_inds(group_inds.cpu().numpy()))
+    with pytest.raises(RuntimeError, match="int64"):
+        ingroup_indices.forward(group_inds, torch.zeros(n, dtype=torch.int32, device=DEV))
+    with pytest.raises(RuntimeError, match="one entry per element"):
+        ingroup_indices.forward(group_inds, torch.zeros(n + 1, dtype=torch.int64, device=DEV))
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        ingroup_indices.forward(group_inds.cpu(), torch.zeros(n, dtype=torch.int64))
+
+
+@pytest.mark.parametrize("B,P,cap,max_all,extra", [
+    (40, 60_000, 512, 50_000, [0.0, 0.0, 0.0]),
+    (7, 1_000, 16, 60, [1.0, 0.2, 0.4]),             # both caps bite
+])
+def test_reference_module_dynamic_point_pool_ext_forward_in_place(B, P, cap, max_all, extra):
+    tx()
+    import dynamic_point_pool_ext
+    rois, pts = _boxes_and_points(B * 11 + P, B, P)
+    rois, pts = rois.to(DEV), pts.to(DEV)
+    say(f"[case] dynamic_point_pool_ext.forward B={B} P={P} cap={cap} max_all={max_all}")
+    out_pts_idx = -1 * pts.new_ones(max_all, dtype=torch.long)          # dynamic_point_pool_op.py:33-35
+    out_roi_idx = -1 * pts.new_ones(max_all, dtype=torch.long)
+    out_pts_feats = pts.new_zeros(max_all, 13, dtype=torch.float)
+    assert dynamic_point_pool_ext.forward(rois, pts, extra, cap, out_pts_idx, out_roi_idx, out_pts_feats) is None
+    valid_mask = out_pts_idx >= 0                                        # :40
+    wi, wr, wf = orc.dynamic_point_pool(rois.cpu().numpy(), pts.cpu().numpy(), extra, cap, max_all)
+    M = wi.shape[0]
+    assert M > 0 and int(valid_mask.sum()) == M and bool(valid_mask[:M].all())   # compact, from index 0
+    assert np.array_equal(out_pts_idx[valid_mask].cpu().numpy(), wi)
+    assert np.array_equal(out_roi_idx[valid_mask].cpu().numpy(), wr)
+    assert np.array_equal(out_pts_feats[valid_mask].cpu().numpy().view(np.uint32), wf.view(np.uint32))
+    # what lies behind the last entry keeps the caller's fill
+    assert (out_roi_idx[M:] == -1).all() and (out_pts_feats[M:] == 0).all()
+    with pytest.raises(RuntimeError, match="13"):
+        dynamic_point_pool_ext.forward(rois, pts, extra, cap, out_pts_idx, out_roi_idx,
+                                       pts.new_zeros(max_all, 12, dtype=torch.float))
+
+
+def test_reference_module_dynamic_point_pool_ext_mixed_in_place():
+    tx()
+    import dynamic_point_pool_ext
+    rois, pts = _boxes_and_points(321, 60, 50_000)
+    g = torch.Generator().manual_seed(5)
+    rb = torch.randint(0, 3, (60,), generator=g).int()
+    pb = torch.randint(0, 3, (50_000,), generator=g).int()
+    extra, cap, max_all = [0.4, 0.4, 0.2], 64, 20_000
+    oi = torch.full((max_all,), -1, dtype=torch.long, device=DEV)
+    orr = torch.full((max_all,), -1, dtype=torch.long, device=DEV)
+    of = torch.zeros((max_all, 13), device=DEV)
+    say("[case] dynamic_point_pool_ext.dynamic_point_pool_mixed_gpu")
+    dynamic_point_pool_ext.dynamic_point_pool_mixed_gpu(rois.to(DEV), rb.to(DEV), pts.to(DEV), pb.to(DEV), extra, cap,
+                                                        oi, orr, of)
+    wi, wr, wf = orc.dynamic_point_pool(rois.numpy(), pts.numpy(), extra, cap, max_all, rb.numpy(), pb.numpy())
+    M = wi.shape[0]
+    assert M > 50 and int((oi >= 0).sum()) == M
+    assert np.array_equal(oi[:M].cpu().numpy(), wi) and np.array_equal(orr[:M].cpu().numpy(), wr)
+    assert np.array_equal(of[:M].cpu().numpy().view(np.uint32), wf.view(np.uint32))
+
+
+def test_reference_module_grid_hash_ext():
+    tx()
+    import grid_hash_ext
+    rng = np.random.default_rng(29)
+    n = 50_000
+    keys = rng.choice(2 ** 30, size=n, replace=False).astype(np.int32)
+    vals = rng.permutation(n).astype(np.int32)
+    say(f"[case] grid_hash_ext n={n}")
+    table = grid_hash_ext.build_table(torch.from_numpy(keys).to(DEV), torch.from_numpy(vals).to(DEV))  # grid_hash.py:31
+    assert table.dtype == torch.int32 and tuple(table.shape) == (65536, 2)
+    queries = np.concatenate([keys[::3], rng.integers(0, 2 ** 30, size=999).astype(np.int32)])
+    out = grid_hash_ext.probe_table(torch.from_numpy(queries).to(DEV), table)                           # :44
+    assert np.array_equal(out.cpu().numpy(), orc.grid_hash_probe(queries, orc.grid_hash_build(keys, vals)))

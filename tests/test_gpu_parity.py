@@ -18,7 +18,7 @@ import pytest
 import torch
 
 from oracle import c_oracle as orc
-from torchex_amd import workloads
+from tests import workloads
 
 pytestmark = pytest.mark.gpu
 

@@ -10,7 +10,7 @@ import numpy as np
 import torch
 
 from tests.conftest import ROOT
-from torchex_amd import workloads
+from tests import workloads
 
 
 def _lib():
@@ -123,6 +123,29 @@ def test_package_surface_matches_reference_exports():
     import scatter_ext
     for name in ["sum", "max", "getPreSum"]:   # torchex/src/scatter/scatter.cpp:66-70
         assert callable(getattr(scatter_ext, name))
+    # the modules the reference's other wrappers import by name, with their functions
+    import dynamic_point_pool_ext   # src/dynamic_point_pool/dynamic_point_pool.cpp:166-169
+    import grid_hash_ext            # src/grid_hash/grid_hash.cpp:115-118
+    import ingroup_indices          # src/ingroup_inds/ingroup_inds.cpp:52-54
+    assert callable(ingroup_indices.forward)
+    assert callable(dynamic_point_pool_ext.forward) and callable(dynamic_point_pool_ext.dynamic_point_pool_mixed_gpu)
+    assert callable(grid_hash_ext.build_table) and callable(grid_hash_ext.probe_table)
+
+
+def test_reference_modules_reject_cpu_tensors():
+    import pytest
+    import dynamic_point_pool_ext
+    import grid_hash_ext
+    import ingroup_indices
+    ids = torch.zeros(4, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        ingroup_indices.forward(ids, torch.zeros_like(ids))
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        dynamic_point_pool_ext.forward(torch.zeros((1, 7)), torch.zeros((5, 3)), [0.0, 0.0, 0.0], 8,
+                                       torch.zeros(9, dtype=torch.int64), torch.zeros(9, dtype=torch.int64),
+                                       torch.zeros((9, 13)))
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        grid_hash_ext.build_table(torch.zeros(4, dtype=torch.int32), torch.zeros(4, dtype=torch.int32))
 
 
 def test_cpu_tensors_are_rejected_not_silently_computed():

@@ -9,7 +9,7 @@ import torch
 
 from oracle import c_oracle as orc
 from oracle import torch_oracle as tor
-from torchex_amd import workloads
+from tests import workloads
 
 
 def bits(a):

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from oracle import c_oracle as orc
-from torchex_amd import workloads
+from tests import workloads
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -97,5 +97,57 @@ def test_resident_table_forward_matches_caller_table_forward():
     assert rc == 4
     lib.txs_status_string.restype = ctypes.c_char_p
     assert b"exceeds" in lib.txs_status_string(4)
+    torch.cuda.synchronize()
+    assert bool((out == 7.0).all())
+
+
+def test_resident_table_forward_allocates_nothing():
+    """Device memory as the driver reports it (free bytes of the GPU) and as torch's
+    allocator reports it stay exactly where they were over a series of calls of the
+    entry point, once its kernels have been loaded by a warm-up call of every operator:
+    a hipMalloc (or a torch allocation) inside the entry point would move one of them.
+    Also: an invalid call returns its status without having queued the clearing kernel
+    (the shared table keeps what it held)."""
+    from torchex_amd import _native
+    import torchex_amd as T
+    lib = _native.cabi()
+    assert lib.txs_resident_table_init() == 0
+    lib.txs_scatter_forward_resident.restype = ctypes.c_int
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    w = workloads.lidar_pillars(N=200_000, C=32, seed=11)
+    f = w.feats.to(DEV)
+    data = T.ScatterData(w.unq_inv.to(DEV), w.unq_cnts.to(DEV))
+    assert data.num_heavy > 0
+    N, C, U = w.N, w.C, w.U
+    vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    out = torch.empty((U, C), device=DEV)
+    arg = torch.empty((U, C), device=DEV, dtype=torch.int32)
+
+    def call(op, dtype=F32):
+        return lib.txs_scatter_forward_resident(
+            ci(op), ci(dtype), vp(f.data_ptr()), vp(data.row_ids.data_ptr()), vp(data.perm.data_ptr()),
+            vp(data.seg.data_ptr()), vp(data.preSum.data_ptr()), vp(data.slot_of.data_ptr()),
+            vp(data.heavy_ids.data_ptr()), i64(data.num_special), i64(data.num_heavy), vp(out.data_ptr()),
+            vp(arg.data_ptr()), i64(N), i64(C), i64(U), i64(data.max_cnt), ci(VOXEL_ORDER), stream)
+
+    _say(f"[case] resident table: no allocation, N={N} C={C} U={U} heavy={data.num_heavy}")
+    for op in (SUM, MEAN, MAX):                      # warm-up: loads every kernel involved
+        assert call(op) == 0
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    alloc0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(5):
+        for op in (SUM, MEAN, MAX):
+            assert call(op) == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, f"free device memory moved by {free0 - free1} bytes"
+    assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+    wm, wa = orc.scatter_max_first(w.feats.numpy(), w.unq_inv.numpy().astype(np.int32), U)
+    assert np.array_equal(arg.cpu().numpy(), wa) and np.array_equal(out.cpu().numpy(), wm)
+    # an unsupported dtype is refused before anything is queued: outputs untouched
+    out.fill_(7.0)
+    torch.cuda.synchronize()
+    assert call(SUM, dtype=9) == 3
     torch.cuda.synchronize()
     assert bool((out == 7.0).all())

@@ -1,4 +1,6 @@
-"""Seeded synthetic inputs for the voxel scatter path.
+"""Seeded synthetic inputs for the voxel scatter path: test and benchmark
+infrastructure (used by the tests, ``bench.py`` and the smoke entry point), not part
+of the product package.
 
 Every workload is generated on the CPU with ``torch.Generator().manual_seed``
 and returned as CPU tensors, so a CPU checker and the GPU kernels see identical

@@ -25,6 +25,11 @@ except ImportError as e:  # pragma: no cover
 # The reference does `import scatter_ext` (torchex/operator_py/scatter_op.py:4);
 # keep that spelling importable.
 sys.modules.setdefault("scatter_ext", scatter_ext)
+# The same for the modules its other wrappers import: `import ingroup_indices`
+# (operator_py/ingroup_inds_op.py:4), `import dynamic_point_pool_ext`
+# (operator_py/dynamic_point_pool_op.py:7), `import grid_hash_ext` (operator_py/grid_hash.py:2).
+for _name in ("ingroup_indices", "dynamic_point_pool_ext", "grid_hash_ext"):
+    sys.modules.setdefault(_name, getattr(scatter_ext, _name))
 
 
 def cabi():

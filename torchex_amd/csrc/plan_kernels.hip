@@ -11,6 +11,8 @@
 
 #include "txs_common.h"
 
+#include <atomic>
+
 namespace {
 
 // -------------------------------------------------------------- small utils --
@@ -903,6 +905,10 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
     }
 }
 
+__global__ void stats_clear_kernel(int *__restrict__ stats) {
+    if (threadIdx.x < TXS_STATS_LEN) stats[threadIdx.x] = 0;
+}
+
 int radix_bits(int64_t U) {
     int bits = 1;
     while ((1LL << bits) < U) ++bits;
@@ -1099,6 +1105,12 @@ int txs_detail::plan_build(const int32_t *unq_inv, int64_t num_total, int64_t nu
     if (((uintptr_t)plan_ws & 7u) != 0) return TXS_ERR_INVALID_ARG;
     if (slot_of == nullptr) heavy_threshold = 0x7fffffff;  // no special voxels: no flag bit in seg
     const int bits = radix_bits(U > 1 ? U : 1);
+    if (n == 0 || U == 0) {
+        // nothing to sort: the general sequence only writes the offsets and the table of
+        // (empty) voxels; it adds to `stats`, which this call promises to initialise itself
+        stats_clear_kernel<<<dim3(1), dim3(64), 0, st>>>(stats);
+        if (hipGetLastError() != hipSuccess) return TXS_ERR_LAUNCH;
+    }
     if (n == 0 || U == 0 || bits > kBucketBitsMax)
         return txs_plan_build_general(unq_inv, num_total, num_unq, heavy_threshold, unq_cnts, plan_ws, perm, seg,
                                       preSum, slot_of, heavy_ids, stats, stream);
@@ -1124,14 +1136,18 @@ int txs_detail::plan_build(const int32_t *unq_inv, int64_t num_total, int64_t nu
     int *wg_pick = reinterpret_cast<int *>(  // 16-byte records
         ((uintptr_t)(scan_ws + scan_tiles(used + 1) + 17) + 15u) & ~(uintptr_t)15u);
     int *part_hist = wg_pick + 4 * groups;
-    static bool lds_allowed = false;
-    if (!lds_allowed) {
+    // (the attribute belongs to the current device's copy of a kernel: once per device)
+    constexpr int kMaxDevices = 64;
+    static std::atomic<bool> lds_allowed[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return TXS_ERR_LAUNCH;
+    if (!lds_allowed[dev].load(std::memory_order_acquire)) {
         for (const void *k : {reinterpret_cast<const void *>(bucket_scatter_kernel<4>),
                               reinterpret_cast<const void *>(bucket_scatter_kernel<8>),
                               reinterpret_cast<const void *>(bucket_scatter_kernel<16>)})
             if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) != hipSuccess)
                 return TXS_ERR_LAUNCH;
-        lds_allowed = true;
+        lds_allowed[dev].store(true, std::memory_order_release);
     }
     auto hist_kernel = items == 16 ? bucket_hist_kernel<16> : (items == 8 ? bucket_hist_kernel<8> : bucket_hist_kernel<4>);
     auto scatter_kernel =

@@ -18,6 +18,7 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <algorithm>
+#include <limits>
 #include <optional>
 #include <tuple>
 #include <utility>
@@ -246,7 +247,12 @@ unique_plan(const Tensor &keys_in, int64_t key_bound, int64_t heavy_threshold, c
         hs[TXS_STAT_NUM_UNQ] = U;
         return {unq.narrow(0, 0, U), inv, cnts, preSum, perm_out, seg, slot_of, heavy_ids, hs};
     }
-    const Tensor keys = keys_in.scalar_type() == at::kInt ? keys_in : keys_in.to(at::kInt);
+    // int64 keys are narrowed for the sort; one outside int32 is first pinned to a value that
+    // stays outside [0, key_bound) (key_bound is below 2^31 - 1), so that the range check on
+    // the device flags it instead of seeing its low 32 bits
+    const Tensor keys = keys_in.scalar_type() == at::kInt
+                            ? keys_in
+                            : keys_in.clamp(-1, (int64_t)std::numeric_limits<int32_t>::max()).to(at::kInt);
     Tensor seg = empty_i32(N, keys), perm = empty_i32(N, keys), inv = empty_i32(N, keys);
     Tensor unq = empty_i32(N, keys), preSum = empty_i32(N + 1, keys);
     Tensor slot_of = empty_i32(N, keys), heavy_all = empty_i32(N, keys);
@@ -295,7 +301,8 @@ Tensor ingroup_inds(const Tensor &seg, const OptTensor &perm, const Tensor &preS
 // with the number of rows as the bound of the ids (true for the inverse of a unique; the
 // largest id is then never read back), the rank kernel, one host synchronisation.  Ids at
 // or above the number of rows take a second pass with their true bound.
-Tensor group_ranks(const Tensor &ids_in) {
+// `out`: int64, contiguous, one entry per id; written in place.
+void group_ranks_into(const Tensor &ids_in, Tensor &out) {
     check_dev(ids_in, "group_inds");
     TORCH_CHECK(ids_in.scalar_type() == at::kInt || ids_in.scalar_type() == at::kLong,
                 "group_inds must be int32 or int64");
@@ -303,8 +310,7 @@ Tensor group_ranks(const Tensor &ids_in) {
     Tensor ids = ids_in.reshape({-1}).contiguous();
     if (ids.scalar_type() != at::kInt) ids = ids.to(at::kInt);
     const int64_t N = ids.numel();
-    Tensor out = at::empty({N}, ids.options().dtype(at::kLong));
-    if (N == 0) return out;
+    if (N == 0) return;
     void *st = cur_stream(ids);
     // `exact`: U is the true bound of the ids (largest id + 1), not the guess `number of rows`
     auto attempt = [&](int64_t U, bool exact) -> bool {
@@ -340,7 +346,27 @@ Tensor group_ranks(const Tensor &ids_in) {
         TORCH_CHECK(lo >= 0, "group_inds must be non-negative");
         TORCH_CHECK(attempt(hi + 1, true), "group_inds could not be ranked");
     }
+}
+
+Tensor group_ranks(const Tensor &ids_in) {
+    check_dev(ids_in, "group_inds");
+    Tensor out = at::empty({ids_in.numel()}, ids_in.options().dtype(at::kLong));
+    group_ranks_into(ids_in, out);
     return out;
+}
+
+// ---- the reference's ingroup_indices module (ingroup_inds.cpp:28-54) --------
+
+// forward(group_inds, out_inds): both int64 and caller-allocated (the wrapper passes
+// zeros_like(group_inds) - 1, ingroup_inds_op.py:15-17); every entry of out_inds is written.
+void ingroup_inds_ref(Tensor group_inds, Tensor out_inds) {
+    check_dev(group_inds, "group_inds");
+    check_dev(out_inds, "out_inds");
+    TORCH_CHECK(group_inds.scalar_type() == at::kLong, "group_inds must be int64, got ", group_inds.scalar_type());
+    TORCH_CHECK(out_inds.scalar_type() == at::kLong, "out_inds must be int64, got ", out_inds.scalar_type());
+    TORCH_CHECK(out_inds.numel() == group_inds.numel(), "out_inds must have one entry per element of group_inds");
+    TORCH_CHECK(out_inds.device() == group_inds.device(), "group_inds and out_inds live on different devices");
+    group_ranks_into(group_inds, out_inds);
 }
 
 // dynamic_point_pool(rois [B,7], pts [P,3], extra_wlh, max_pts_per_box, max_all_pts)
@@ -384,6 +410,67 @@ std::tuple<Tensor, Tensor, Tensor> dynamic_point_pool(const Tensor &rois, const 
                  "dynamic_point_pool");
     const int64_t M = num.cpu().data_ptr<int32_t>()[0];
     return {idx.narrow(0, 0, M), roi.narrow(0, 0, M), feats.narrow(0, 0, M)};
+}
+
+// ---- the reference's dynamic_point_pool_ext module (dynamic_point_pool.cpp:58-169) ----
+
+// The outputs come from the caller (the wrapper fills them with -1 / -1 / 0,
+// dynamic_point_pool_op.py:33-35), max_all_pts is their length, and the entries are
+// written from index 0 on; what lies behind the last entry keeps the caller's fill.  No
+// host synchronisation (the reference reads its counter back between its two kernels).
+void dpp_into(const Tensor &rois, const OptTensor &rois_batch, const Tensor &pts, const OptTensor &pts_batch,
+              const std::vector<double> &extra_wlh, int64_t max_pts_per_box, Tensor &out_pts_idx,
+              Tensor &out_roi_idx, Tensor &out_pts_feats) {
+    check_dev(rois, "rois");
+    check_dev(pts, "pts");
+    check_dev(out_pts_idx, "out_pts_idx");
+    check_dev(out_roi_idx, "out_roi_idx");
+    check_dev(out_pts_feats, "out_pts_feats");
+    TORCH_CHECK(rois.dim() == 2 && rois.size(1) == 7 && rois.scalar_type() == at::kFloat,
+                "rois must be float32 [num_boxes, 7]");
+    TORCH_CHECK(pts.dim() == 2 && pts.size(1) == 3 && pts.scalar_type() == at::kFloat,
+                "pts must be float32 [num_pts, 3]");
+    TORCH_CHECK(extra_wlh.size() == 3, "extra_wlh needs 3 entries");
+    TORCH_CHECK(max_pts_per_box >= 0, "max_num_pts_per_box must be non-negative");
+    const int64_t B = rois.size(0), P = pts.size(0), M = out_pts_idx.size(0);
+    TORCH_CHECK(out_pts_idx.scalar_type() == at::kLong && out_pts_idx.dim() == 1, "out_pts_idx must be int64 [max_all_pts]");
+    TORCH_CHECK(out_roi_idx.scalar_type() == at::kLong && out_roi_idx.dim() == 1 && out_roi_idx.size(0) == M,
+                "out_roi_idx must be int64 [max_all_pts]");
+    TORCH_CHECK(out_pts_feats.scalar_type() == at::kFloat && out_pts_feats.dim() == 2 && out_pts_feats.size(0) == M &&
+                    out_pts_feats.size(1) == 13,
+                "out_pts_feats must be float32 [max_all_pts, 13]");  // info_dim == 13, dynamic_point_pool.cpp:80-81
+    if (rois_batch.has_value()) {
+        check_i32(*rois_batch, "rois_batch");
+        check_i32(*pts_batch, "pts_batch");
+        TORCH_CHECK(rois_batch->numel() == B, "rois_batch must be [num_boxes]");
+        TORCH_CHECK(pts_batch->numel() == P, "pts_batch must be [num_pts]");
+    }
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(pts.device());
+    const float extra[3] = {(float)extra_wlh[0], (float)extra_wlh[1], (float)extra_wlh[2]};
+    auto iopt = pts.options().dtype(at::kInt);
+    Tensor ws = at::empty({txs_dpp_workspace_len(P, B) + 2}, iopt);
+    Tensor num = at::zeros({1}, iopt);
+    check_status(txs_dynamic_point_pool_mixed(B ? rois.data_ptr<float>() : nullptr, opt_i32p(rois_batch),
+                                              P ? pts.data_ptr<float>() : nullptr, opt_i32p(pts_batch), B, P, extra,
+                                              (int32_t)max_pts_per_box, M, i32w(ws),
+                                              M ? out_pts_idx.data_ptr<int64_t>() : nullptr,
+                                              M ? out_roi_idx.data_ptr<int64_t>() : nullptr,
+                                              M ? out_pts_feats.data_ptr<float>() : nullptr, i32w(num), cur_stream(pts)),
+                 "dynamic_point_pool");
+}
+
+// forward(rois, pts, extra_wlh, max_num_pts_per_box, out_pts_idx, out_roi_idx, out_pts_feats)
+void dpp_forward_ref(Tensor rois, Tensor pts, std::vector<double> extra_wlh, int64_t max_num_pts_per_box,
+                     Tensor out_pts_idx, Tensor out_roi_idx, Tensor out_pts_feats) {
+    dpp_into(rois, std::nullopt, pts, std::nullopt, extra_wlh, max_num_pts_per_box, out_pts_idx, out_roi_idx,
+             out_pts_feats);
+}
+
+// dynamic_point_pool_mixed_gpu(rois, rois_batch, pts, pts_batch, extra_wlh, max_num_pts_per_box, out...)
+void dpp_mixed_ref(Tensor rois, Tensor rois_batch, Tensor pts, Tensor pts_batch, std::vector<double> extra_wlh,
+                   int64_t max_num_pts_per_box, Tensor out_pts_idx, Tensor out_roi_idx, Tensor out_pts_feats) {
+    dpp_into(rois, rois_batch, pts, pts_batch, extra_wlh, max_num_pts_per_box, out_pts_idx, out_roi_idx,
+             out_pts_feats);
 }
 
 int64_t up_2n_host(int64_t n) {  // torchex/src/grid_hash/grid_hash.cpp:28-37
@@ -627,6 +714,7 @@ struct CsrPlan {
     explicit CsrPlan(const Tensor &preSum) : owner(preSum.getIntrusivePtr()) {}
 };
 constexpr size_t kCsrPlanCacheSize = 8;
+constexpr size_t kCsrPlanScratchKept = 4;
 std::vector<CsrPlan> &csr_plan_cache() {
     // touched under the GIL only; never destroyed, so no device tensor is freed after
     // the runtime has shut down at interpreter exit
@@ -703,6 +791,8 @@ void csr_reduce(int op, Tensor feats, Tensor preSum, Tensor out, OptTensor arg, 
             if (std::get<0>(entry) == C && std::get<1>(entry) == st) scratch = std::get<2>(entry);
         if (!scratch.defined()) {
             scratch = make_scratch(feats.size(0), C, preSum.numel() - 1, plan.num_heavy, feats);
+            // the newest few are kept: a table can hold tens of MB of partial tables
+            if (plan.scratch.size() >= kCsrPlanScratchKept) plan.scratch.erase(plan.scratch.begin());
             plan.scratch.emplace_back(C, st, scratch);
         }
         seg = plan.seg;
@@ -806,4 +896,20 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.attr("MEAN") = (int)TXS_MEAN;
     m.attr("MAX") = (int)TXS_MAX;
     m.attr("MAX_REFTIE") = (int)TXS_MAX_REFTIE;
+
+    // The reference's other three extension modules, with their own names and positional
+    // signatures, so that operator_py/ingroup_inds_op.py, dynamic_point_pool_op.py and
+    // grid_hash.py bind as they are (torchex_amd/_native.py registers them in sys.modules).
+    auto ig = m.def_submodule("ingroup_indices", "the reference's ingroup_indices module (ingroup_inds.cpp:52-54)");
+    ig.def("forward", &ingroup_inds_ref, "forward(group_inds, out_inds): rank of every element inside its group, in place");
+    auto dp = m.def_submodule("dynamic_point_pool_ext",
+                              "the reference's dynamic_point_pool_ext module (dynamic_point_pool.cpp:166-169)");
+    dp.def("forward", &dpp_forward_ref,
+           "forward(rois, pts, extra_wlh, max_num_pts_per_box, out_pts_idx, out_roi_idx, out_pts_feats), in place");
+    dp.def("dynamic_point_pool_mixed_gpu", &dpp_mixed_ref,
+           "dynamic_point_pool_mixed_gpu(rois, rois_batch, pts, pts_batch, extra_wlh, max_num_pts_per_box, "
+           "out_pts_idx, out_roi_idx, out_pts_feats), in place");
+    auto gh = m.def_submodule("grid_hash_ext", "the reference's grid_hash_ext module (grid_hash.cpp:115-118)");
+    gh.def("build_table", &grid_hash_build, "build_table(coors, values) -> table");
+    gh.def("probe_table", &grid_hash_probe, "probe_table(coors, table) -> values");
 }

@@ -849,13 +849,22 @@ const int32_t *row_order_ids(const int32_t *unq_inv, const int32_t *perm, const 
     return unq_inv ? unq_inv : (perm == nullptr ? seg : nullptr);
 }
 
+__global__ void clear_cells_kernel(unsigned long long *__restrict__ cells, long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) cells[i] = 0ull;
+}
+
 // Argument checks, the choice between the row-order table kernels and the voxel-order
 // kernels, and the launches, behind txs_scatter_forward and txs_scatter_forward_resident.
+// clear_heavy_cells: the heavy voxels' cells of `scratch` may hold anything on entry (the
+// library-resident table); they are cleared by a kernel once the arguments have passed
+// every check and only if the voxel-order kernels, which use them, are the ones that run.
 int scatter_forward_impl(int op, int dtype, const void *feats, const int32_t *unq_inv, const int32_t *perm,
                          const int32_t *seg, const int32_t *preSum, const int32_t *slot_of,
                          const int32_t *heavy_ids, int64_t num_special, int64_t num_heavy, void *scratch,
                          int64_t scratch_cells, void *out, int32_t *arg, int64_t num_total, int64_t channel,
-                         int64_t num_unq, int64_t max_cnt, int path, void *stream) {
+                         int64_t num_unq, int64_t max_cnt, int path, void *stream,
+                         bool clear_heavy_cells = false) {
     if (op != TXS_SUM && op != TXS_MEAN && op != TXS_MAX && op != TXS_MAX_REFTIE)
         return TXS_ERR_UNSUPPORTED;
     if (dtype != TXS_F32 && dtype != TXS_F16 && dtype != TXS_BF16) return TXS_ERR_UNSUPPORTED;
@@ -892,6 +901,11 @@ int scatter_forward_impl(int op, int dtype, const void *feats, const int32_t *un
     if (num_special > 0 && !heavy_ids) return TXS_ERR_INVALID_ARG;
     const int elem = dtype == TXS_F32 ? 4 : 2;
     hipError_t e = hipSuccess;
+    if (clear_heavy_cells && heavy_cells > 0) {
+        clear_cells_kernel<<<dim3(blocks_for(heavy_cells)), dim3(kThreads), 0, st>>>(
+            static_cast<unsigned long long *>(scratch), heavy_cells);
+        if (hipGetLastError() != hipSuccess) return TXS_ERR_LAUNCH;
+    }
     if (N > 0) {
         Geometry geo = make_geometry(N, C, elem, feats, out, nullptr, is_max, arg, fwd_chunk_for(N, U, op, elem));
         if (dtype == TXS_F32)
@@ -1051,11 +1065,6 @@ int resident_table(unsigned long long **table) {
     return TXS_OK;
 }
 
-__global__ void clear_cells_kernel(unsigned long long *__restrict__ cells, long n) {
-    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) cells[i] = 0ull;
-}
-
 }  // namespace
 
 extern "C" {
@@ -1080,15 +1089,12 @@ int txs_scatter_forward_resident(int op, int dtype, const void *feats, const int
     unsigned long long *table = nullptr;
     const int rc = resident_table(&table);
     if (rc != TXS_OK) return rc;
-    if (cells > 0) {
-        // the table is shared by every call on this GPU and keeps what the last one left:
-        // clear the part the heavy voxels use (a kernel, so that the call can be captured)
-        clear_cells_kernel<<<dim3(blocks_for(cells)), dim3(kThreads), 0, (hipStream_t)stream>>>(table, cells);
-        if (hipGetLastError() != hipSuccess) return TXS_ERR_LAUNCH;
-    }
+    // the table is shared by every call on this GPU and keeps what the last one left: the
+    // part the heavy voxels use is cleared (by a kernel, so that the call can be captured)
+    // after the argument checks, and only when the kernels that use it are launched
     return scatter_forward_impl(op, dtype, feats, unq_inv, perm, seg, preSum, slot_of, heavy_ids, num_special,
                                 num_heavy, table, kResidentCells, out, arg, num_total, channel, num_unq,
-                                max_cnt, path, stream);
+                                max_cnt, path, stream, /*clear_heavy_cells=*/true);
 }
 
 }  // extern "C"

@@ -17,6 +17,8 @@
 
 #include "txs_common.h"
 
+#include <atomic>
+
 namespace {
 
 constexpr int kTableThreads = 1024;          // one workgroup per compute unit
@@ -316,27 +318,40 @@ __global__ __launch_bounds__(kTableThreads) void table_bwd_kernel(
 
 // ------------------------------------------------------------------- launch --
 
-int table_workgroups(long N) {
-    static int cus = 0;  // compute units of the current device
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            cus = 256;
+// Compute units of the current device (looked up once per device and kept: the only state
+// this translation unit holds besides the per-kernel "large LDS allowed" flags).
+constexpr int kMaxDevices = 64;
+int compute_units() {
+    static std::atomic<int> cus[kMaxDevices];  // 0 = not asked yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev].store(n, std::memory_order_relaxed);  // every thread that races here stores the same value
     }
+    return n;
+}
+
+int table_workgroups(long N) {
+    const int cus = compute_units();
     // at least 4096 rows per workgroup: a partial table costs as much as its rows otherwise
     long w = (N + 4095) / 4096;
     const long most = cus < TXS_TABLE_MAX_WGS ? cus : TXS_TABLE_MAX_WGS;
     return (int)(w < 1 ? 1 : (w > most ? most : w));
 }
 
+// Tables above 64 KB need the kernel's dynamic-LDS limit raised; the attribute belongs to the
+// current device's copy of the kernel, so it is set once per (instantiation, device).
 template <class K>
-hipError_t allow_lds(K kernel, unsigned bytes) {
-    if (bytes <= 64 * 1024) return hipSuccess;
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+hipError_t allow_lds(K kernel, std::atomic<bool> (&done)[kMaxDevices]) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    if (done[dev].load(std::memory_order_acquire)) return hipSuccess;
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, kTableLdsBudget);
+    if (e == hipSuccess) done[dev].store(true, std::memory_order_release);
+    return e;
 }
 
 template <class TR, int VEC, int OP>
@@ -345,11 +360,8 @@ hipError_t launch_table_fwd(const txs_detail::TablePlan &tp, hipStream_t st, con
                             int N, int C, int U) {
     using raw = typename TR::raw;
     auto kernel = table_fwd_kernel<TR, VEC, OP>;
-    static bool lds_allowed = false;  // per instantiation; the attribute is set for the largest table
-    if (!lds_allowed) {
-        if (allow_lds(kernel, kTableLdsBudget) != hipSuccess) return hipErrorInvalidValue;
-        lds_allowed = true;
-    }
+    static std::atomic<bool> lds_allowed[kMaxDevices];  // per instantiation and device
+    if (allow_lds(kernel, lds_allowed) != hipSuccess) return hipErrorInvalidValue;
     kernel<<<dim3(tp.workgroups), dim3(kTableThreads), tp.lds_bytes, st>>>(
         (const raw *)feats, inv, partials, N, C, U, tp.lpr_log2, tp.stride, tp.rows_per_wg);
     const long total = (long)U * C;
@@ -375,11 +387,8 @@ hipError_t launch_table_bwd(const txs_detail::TablePlan &tp, hipStream_t st, con
                             const int *inv, const int *preSum, void *gin, int N, int C, int U) {
     using raw = typename TR::raw;
     auto kernel = table_bwd_kernel<TR, VEC, OP>;
-    static bool lds_allowed = false;
-    if (!lds_allowed) {
-        if (allow_lds(kernel, kTableLdsBudget) != hipSuccess) return hipErrorInvalidValue;
-        lds_allowed = true;
-    }
+    static std::atomic<bool> lds_allowed[kMaxDevices];
+    if (allow_lds(kernel, lds_allowed) != hipSuccess) return hipErrorInvalidValue;
     kernel<<<dim3(tp.workgroups), dim3(kTableThreads), tp.lds_bytes, st>>>(
         (const raw *)g, arg, inv, preSum, (raw *)gin, N, C, U, tp.lpr_log2, tp.stride, tp.rows_per_wg);
     return hipGetLastError();

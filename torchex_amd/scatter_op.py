@@ -44,6 +44,9 @@ def _resolve_tie_rule(rule, grouped):
     return rule
 
 
+_SCRATCH_KEPT = 4   # forward workspaces a ScatterData keeps (most recently used)
+
+
 class ScatterData:
     """Index bundle shared by the scatter operators (``scatter_op.py:7-21``).
 
@@ -152,14 +155,20 @@ class ScatterData:
     def scratch(self, channel):
         """Forward workspace: the zeroed table the heavy voxels are merged in (one row each,
         left zeroed again by the kernels) and, for inputs with few voxels, room for the
-        partial tables of the row-order kernels.  A buffer is kept for reuse -- one per
-        channel count and per stream: calls queued on one stream are ordered, and forwards
-        that run concurrently on different streams each get a workspace of their own."""
+        partial tables of the row-order kernels.  Buffers are kept for reuse -- one per
+        channel count and per stream (calls queued on one stream are ordered, and forwards
+        that run concurrently on different streams each get a workspace of their own), the
+        ``_SCRATCH_KEPT`` most recently used at most."""
         key = (channel, torch.cuda.current_stream(self.seg.device).stream_id)
-        buf = self._scratch.get(key)
+        buf = self._scratch.pop(key, None)
         if buf is None:
             buf = scatter_ext.make_scratch(self.num_total, channel, self.num_unq, self.num_heavy, self.seg)
-            self._scratch[key] = buf
+            # the few most recently used are kept (a buffer can hold tens of MB of partial
+            # tables); one that is dropped was only ever used on its own stream, so the
+            # allocator may hand its memory on as soon as that stream's queued work allows
+            while len(self._scratch) >= _SCRATCH_KEPT:
+                self._scratch.pop(next(iter(self._scratch)))
+        self._scratch[key] = buf          # most recently used last
         return buf
 
     def forward_args(self, channel):
