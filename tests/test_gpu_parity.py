@@ -1230,7 +1230,18 @@ def test_element_offsets_beyond_2_to_31():
         out, out_t = (res[0], res_t[0]) if name == "max" else (res, res_t)
         # singletons: the voxel's row itself (sum of one, mean over one, max of one)
         assert same_bits(out[:H].index_select(0, head_ids), feats[:H].detach()), f"{name}: singleton rows"
-        assert same_bits(out[H:], out_t), f"{name}: voxels of the rows past element 2^31"
+        if name == "max":
+            assert same_bits(out[H:], out_t), f"{name}: voxels of the rows past element 2^31"
+        else:
+            # a voxel whose rows straddle two lane groups' chunks is summed as (earlier part) +
+            # (later part), and where the chunk borders fall depends on the rows in front: the
+            # fp32 sums of the two problems can differ in their last bit, which reaches the
+            # fp16 output in a handful of the 12.8 M elements (by one unit in the last place)
+            a, b = out[H:].detach().float(), out_t.detach().float()
+            both_nan = torch.isnan(a) & torch.isnan(b)
+            differs = (out[H:].contiguous().view(torch.int16) != out_t.contiguous().view(torch.int16)) & ~both_nan
+            assert int(differs.sum()) <= 64, f"{name}: {int(differs.sum())} elements differ"
+            assert torch.allclose(a, b, rtol=2.0 ** -10, atol=2.0 ** -24, equal_nan=True), f"{name}: rows past element 2^31"
         if name == "max":
             arg, arg_t = res[1], res_t[1]
             assert torch.equal(arg[:H].index_select(0, head_ids),

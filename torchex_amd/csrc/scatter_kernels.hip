@@ -88,208 +88,269 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     int lpr_log2, int ref_log2) {
     using raw = typename TR::raw;
     constexpr bool kMax = OP == TXS_MAX || OP == TXS_MAX_REFTIE;
+    constexpr bool kRef = OP == TXS_MAX_REFTIE;  // idx[] then holds the winner's staged position, not its row
     // (the fp16 running max keeps packed halves and has registers to spare for a deeper batch)
     constexpr int kBatch = sizeof(raw) == 2 ? ((kMax && std::is_same<TR, F16>::value) ? kBatchHalfMax : kBatchHalf) : ::kBatch;
-    constexpr bool kRef = OP == TXS_MAX_REFTIE;  // idx[] then holds the winner's staged position, not its row
+    using AccT = typename std::conditional<kMax, typename TR::max_t, float>::type;
+    constexpr int kEndBit = kSpecialBit;
     extern __shared__ int lds[];
-    const int G = kThreads >> lpr_log2;
+    const int g_log2 = 8 - lpr_log2;      // kThreads == 256
+    const int G = 1 << g_log2;
     const int T = G * CHUNK;
     const int n_seg_s = T + kMargin + 1;  // positions t0-1 .. t0+T+kMargin-1
-    int *seg_s = lds;
-    int *perm_s = lds + n_seg_s;          // positions t0 .. t0+T+kMargin-1
-    // Partials of heavy voxels: two slots per lane group (a chunk can touch at
-    // most two heavy runs, one at each end), combined across the workgroup
-    // before anything goes to the global scratch table.
-    // (sum / mean partials are parked as doubles: LDS fp64 atomic adds run several times
-    // faster than fp32 ones on this part)
-    using SlotT = typename std::conditional<kMax, unsigned long long, double>::type;
-    int *slot_id = perm_s + (n_seg_s - 1);
-    SlotT *slot_val = reinterpret_cast<SlotT *>(lds + ((2 * n_seg_s - 1 + 2 * G + 1) & ~1));
-    const int W = VEC << lpr_log2;        // elements per slot
+    int *seg_s = lds;                     // seg_s[l]: voxel (bit 31: special) at position t0 - 1 + l
+    int *pk_s = lds + n_seg_s;            // pk_s[l - 1]: row at position t0 - 1 + l, bit 31 = last row of its run
+    int *bnd_s = lds + 2 * n_seg_s - 1;   // [0]: first l of the tile's own range, [1]: one past its last l
+    // what a lane group hands to the next one: the reduction of the run that is still open at
+    // the end of its share (4-byte cells: a value per element, and for max the winner's tag)
+    float *carry_v = reinterpret_cast<float *>(lds + ((2 * n_seg_s + 1 + 3) & ~3));
+    int *carry_i = reinterpret_cast<int *>(carry_v) + kThreads * VEC;
     const long t0l = (long)xcd_block(blockIdx.x, gridDim.x) * T;
     if (t0l >= N) return;  // uniform for the workgroup
     const int t0 = (int)t0l;
-    bool saw_heavy = false;
-    for (int e = threadIdx.x; e < n_seg_s; e += kThreads) {
+    const unsigned last_row = (unsigned)(N - 1);
+
+    // Stage the tile's ids.  The tile's own range [b_lo, b_hi) starts at the first position
+    // at or after the tile's first one where a run starts (or that lies in a heavy run, which
+    // is split anywhere) and ends at the first such position at or after the next tile's first
+    // one: an ordinary run belongs, whole, to the tile it starts in.  Both are found among the
+    // kMargin positions behind each border with one wave ballot.
+    for (int e0 = 0; e0 < n_seg_s; e0 += kThreads) {
+        const int e = e0 + (int)threadIdx.x;
         const long p = (long)t0 - 1 + e;
-        const bool in = p >= 0 && p < N;
+        const bool in = e < n_seg_s && p >= 0 && p < N;
         const int sv = in ? seg[p] : kNoSeg;
-        seg_s[e] = sv;
-        saw_heavy |= (sv < 0) && e >= 1 && e <= T;  // special bit on a position of this tile
-        if (e >= 1) perm_s[e - 1] = in ? (perm ? perm[p] : (int)p) : -1;
+        const int sn = (e < n_seg_s && p + 1 < N) ? seg[p + 1] : kNoSeg;
+        if (e < n_seg_s) {
+            seg_s[e] = sv;
+            if (e >= 1) {
+                // a row index outside the matrix (only a corrupt plan has one) is clamped
+                const int r = in ? (int)min((unsigned)(perm ? perm[p] : (int)p), last_row) : 0;
+                pk_s[e - 1] = r | ((in && sn != sv) ? kEndBit : 0);
+            }
+        }
+        // position p + 1 (l = e + 1) can open a range: a run starts there, or it is heavy
+        const int eb = e0 + ((int)threadIdx.x & ~63);  // first entry of this wave in this round
+        if (eb == 0 || eb == T) {
+            const unsigned long long m = __ballot(e < n_seg_s && (sn != sv || (sn < 0)));
+            if (((int)threadIdx.x & 63) == 0)
+                bnd_s[eb == 0 ? 0 : 1] = m ? eb + 1 + (int)__builtin_ctzll(m) : -1;
+        }
     }
-    for (int e = threadIdx.x; e < 2 * G; e += kThreads) slot_id[e] = -1;
-    // one barrier publishes the staged indices and tells the whole workgroup
-    // whether the tile touches a heavy voxel (only then is there a merge phase)
-    const bool tile_has_heavy = __syncthreads_or(saw_heavy);
+    __syncthreads();
+    int b_lo = bnd_s[0], b_hi = bnd_s[1];
+    const int l_staged_end = n_seg_s;  // one past the last staged l
+    if (b_lo < 0) {
+        // an ordinary run of more than kMargin rows covers the tile's first positions (only a
+        // plan with a heavy threshold above kMargin has one): look for its end one by one
+        b_lo = kMargin + 1;
+        while (b_lo < l_staged_end && seg_s[b_lo] == seg_s[b_lo - 1] && seg_s[b_lo] >= 0) ++b_lo;
+    }
+    // no border found behind the tile's end: the range ends with the staged ids, and the last
+    // lane group walks on from there, one row at a time
+    const bool long_tail = b_hi < 0;
+    if (long_tail) b_hi = l_staged_end;
+    if (b_lo > b_hi) b_lo = b_hi;
+    const int Tp = b_hi - b_lo;  // rows of the tile's own range: dealt evenly to the lane groups
+    if (Tp <= 0) return;         // uniform for the workgroup
 
     const int gi = (int)threadIdx.x >> lpr_log2;
     const int lane_in = (int)threadIdx.x & ((1 << lpr_log2) - 1);
     const int col = ((int)blockIdx.y << lpr_log2 | lane_in) * VEC;
-    int n_heavy = 0;  // heavy partials this lane group has parked in LDS
+    const bool live = col < C;
+    auto share_begin = [&](int k) -> int { return b_lo + (int)(((long)k * Tp) >> g_log2); };
+    const int c0 = share_begin(gi), c_end = share_begin(gi + 1);  // this lane group's positions (l)
+    const int ch = (Tp + G - 1) >> g_log2;                          // the largest share
 
-    auto reduce_chunk = [&]() {
-    if (col >= C) return;
-    // l indexes seg_s (position t0 - 1 + l); entries past the staged range are
-    // fetched from global memory (only an ordinary run longer than kMargin that
-    // crosses the tile's end gets there)
+    // ids / rows past the staged range are fetched from global memory (only an ordinary run
+    // longer than kMargin that crosses the tile's end gets there)
     auto seg_at = [&](int l) -> int {
         if (l < n_seg_s) return seg_s[l];
         const long p = (long)t0 - 1 + l;
         return p < N ? seg[p] : kNoSeg;
     };
-    auto row_at = [&](int l) -> int {
-        if (l < n_seg_s) return perm_s[l - 1];
+    auto pk_at = [&](int l) -> int {
+        if (l < n_seg_s) return pk_s[l - 1];
         const long p = (long)t0 - 1 + l;
-        return p < N ? (perm ? perm[p] : (int)p) : -1;
+        if (p >= N) return 0;
+        const int r = (int)min((unsigned)(perm ? perm[p] : (int)p), last_row);
+        const int sn = p + 1 < N ? seg[p + 1] : kNoSeg;
+        return r | (sn != seg[p] ? kEndBit : 0);
     };
-
-    // Range [la, lb) this lane group reduces: its chunk, minus the tail of an
-    // ordinary run that began in an earlier chunk, plus the tail of an ordinary
-    // run that begins here and ends later.
-    int la = gi * CHUNK + 1;
-    const int lend = min(la + CHUNK, N - t0 + 1);
-    if (la >= lend) return;
-    {
-        const int s0 = seg_s[la];
-        if (s0 >= 0 && seg_s[la - 1] == s0) {
-            do ++la; while (la < lend && seg_s[la] == s0);
-            if (la >= lend) return;
-        }
-    }
-    int lb = lend;
-    {
-        const int sl = seg_s[lend - 1];
-        if (sl >= 0)
-            while (seg_at(lb) == sl) ++lb;  // ends at the latest at N (kNoSeg)
-    }
-    const int lb_fast = min(lb, n_seg_s);  // end of the part whose ids are staged in LDS
 
     // Start value of a running max: -inf, or in reference-tie mode the
     // reference's own -FLT_MAX (scatter_kernel.cu:139), which -inf never beats.
-    using AccT = typename std::conditional<kMax, typename TR::max_t, float>::type;
     const AccT acc0 = kRef ? (AccT)TR::to_m(TR::lowest()) : (AccT)(kMax ? -__builtin_inff() : 0.0f);
-    // offset of position l inside its voxel, for the reference's tie key; an
-    // ordinary run always starts inside the range, a heavy one may not
-    auto rel_of_run_start = [&](int sg, int l) -> int {
-        if (!kRef || sg >= 0) return 0;
-        const int u = sg & kIdMask;
-        return ((unsigned)u < (unsigned)U) ? (t0 - 1 + l) - preSum[u] : 0;
-    };
-    AccT acc[VEC];
-    int idx[VEC];
-    int cur = seg_s[la];
-    int run_l0 = la;
-    int rel0 = rel_of_run_start(cur, la);
+    AccT acc[VEC], hacc[VEC];
+    int idx[VEC], hidx[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; ++k) {
         acc[k] = acc0;
         idx[k] = -1;
+        hacc[k] = acc0;
+        hidx[k] = -1;
     }
+    int run_l0 = c0;  // first position (of this lane group) of the run being reduced
+    // The first run end in the share closes a run that began in an earlier share unless a run
+    // starts exactly at the share's first position: its reduction is kept (`hacc`) until the
+    // earlier lane groups have published theirs.
+    bool pend_head = c0 < c_end && seg_s[c0 - 1] == seg_s[c0];
+    int head_seg = kNoSeg;  // voxel (with its special bit) of the kept head, kNoSeg: none
+    int head_l = 0;         // its last position
 
+    const char *lane_base = reinterpret_cast<const char *>(feats) + (size_t)col * sizeof(raw);
+    const unsigned row_bytes = (unsigned)C * (unsigned)sizeof(raw);
+    auto row_ptr = [&](int r) -> const raw * {
+        return reinterpret_cast<const raw *>(lane_base + (unsigned long long)(unsigned)r * row_bytes);
+    };
+
+    // tie key of the reference for the row at position l (as staged) of voxel u (reference-tie mode)
+    auto ref_key_at = [&](int l, int u) -> unsigned {
+        return (unsigned)ref_key((t0 - 1 + l) - preSum[u], ref_log2);
+    };
     // What competes in the low word of a heavy voxel's packed key (smaller wins): the row, or in
     // reference-tie mode the reference's tie key of the winner's offset inside its voxel.
-    auto low_word = [&](int id) -> unsigned {
-        return kRef ? (unsigned)ref_key(rel0 + (id - run_l0), ref_log2) : (unsigned)id;
-    };
-    // Emit the finished run [run_l0, run_end) of voxel `cur`.
-    auto flush = [&](int run_end) {
-        const int u = cur & kIdMask;
+    auto low_word = [&](int id, int u) -> unsigned { return kRef ? ref_key_at(id, u) : (unsigned)id; };
+
+    // Write out the finished reduction (a, ix) of voxel sgv: an output row for an ordinary voxel
+    // (cnt rows, all of them reduced here), one atomic per element into the table for a heavy one
+    // (rows [p_lo, p_hi) of the sorted order went into it).  `staged`: every position involved
+    // has its ids in LDS (so no value that the common path uses comes from a global load, which
+    // would make the path wait for every row still on its way).
+    auto emit = [&](auto staged, int sgv, AccT(&a)[VEC], int(&ix)[VEC], int cnt, long p_lo, long p_hi) {
+        constexpr bool kStaged = decltype(staged)::value;
+        const int u = sgv & kIdMask;
         if ((unsigned)u >= (unsigned)U) return;
         if (kMax && !kRef) {
             bool missing = false;
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) missing |= idx[k] < 0;
+            for (int k = 0; k < VEC; ++k) missing |= ix[k] < 0;
             if (__builtin_expect(missing, 0)) {
-                // No value above -inf was seen in some channel: the run holds
-                // only -inf and NaN there.  The first -inf row wins.
-                for (int p = run_l0; p < run_end; ++p) {
-                    const int row = row_at(p);
+                // No value above -inf was seen in some channel: the rows hold only -inf and NaN
+                // there.  The first -inf row wins.
+                // (an ordinary voxel: all its rows; a heavy one: its rows inside [p_lo, p_hi))
+                long lo = preSum[u], hi = preSum[u + 1];
+                if (sgv < 0) {
+                    lo = lo > p_lo ? lo : p_lo;
+                    hi = hi < p_hi ? hi : p_hi;
+                }
+                for (long p = lo; p < hi; ++p) {
+                    const int row = perm ? perm[p] : (int)p;
                     if ((unsigned)row >= (unsigned)N) continue;
                     Pack<raw, VEC> x = ld<raw, VEC>(feats + (size_t)row * C + col);
 #pragma unroll
                     for (int k = 0; k < VEC; ++k)
-                        if (idx[k] < 0 && TR::to_f(x.v[k]) == -__builtin_inff()) idx[k] = row;
+                        if (ix[k] < 0 && TR::to_f(x.v[k]) == -__builtin_inff()) ix[k] = row;
                 }
             }
         }
-        if (cur >= 0) {  // ordinary voxel: the whole run was reduced here
+        if (sgv >= 0) {
             const size_t o = (size_t)u * C + col;
             Pack<raw, VEC> r;
             if (OP == TXS_SUM) {
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) r.v[k] = TR::from_f(acc[k]);
+                for (int k = 0; k < VEC; ++k) r.v[k] = TR::from_f((float)a[k]);
             } else if (OP == TXS_MEAN) {
-                const float d = (float)(run_end - run_l0);
+                const float d = (float)cnt;
+                if constexpr (TXS_FAST_DIV_HALF && sizeof(raw) == 2) {
+                    // 2-byte outputs: the fp32 quotient is rounded to 8 or 11 bits right away, so
+                    // the hardware reciprocal (1 ulp) and one multiply stand in for the division
+                    // (a dozen instructions per element, in a kernel bound by instruction issue)
+                    // (the instruction is spelled out: left to itself the compiler takes a different
+                    // reciprocal instruction where it sees the count come straight from an integer,
+                    // and the two do not always agree in the last bit)
+                    float rd;
+                    asm("v_rcp_f32 %0, %1" : "=v"(rd) : "v"(d));
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) r.v[k] = TR::from_f(acc[k] / d);
+                    for (int k = 0; k < VEC; ++k) {
+                        // (the fp32 product is pinned in a register: where the compiler may fuse the
+                        // multiply with the conversion it rounds once instead of twice, and a sum on
+                        // a rounding boundary would come out differently from one code path to the next)
+                        float q = (float)a[k] * rd;
+                        asm("" : "+v"(q));
+                        r.v[k] = TR::from_f(q);
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) r.v[k] = TR::from_f((float)a[k] / d);
+                }
             } else {
                 Pack<int, VEC> ai;
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) {
-                    r.v[k] = idx[k] >= 0 ? TR::from_m(acc[k]) : TR::lowest();
-                    ai.v[k] = idx[k];
-                    if (kRef && idx[k] >= 0) ai.v[k] = row_at(idx[k]);
+                    r.v[k] = ix[k] >= 0 ? TR::from_m((typename TR::max_t)a[k]) : TR::lowest();
+                    ai.v[k] = ix[k];
+                    if (kRef && ix[k] >= 0) ai.v[k] = (kStaged ? pk_s[ix[k] - 1] : pk_at(ix[k])) & kIdMask;
                 }
                 st_stream<int, VEC>(arg + o, ai);
             }
             st_stream<raw, VEC>(out + o, r);
-        } else if (n_heavy < 2) {  // heavy voxel: park this chunk's partial in LDS
-            const int sidx = 2 * gi + n_heavy;
-            ++n_heavy;
-            if (lane_in == 0) slot_id[sidx] = u;
-            SlotT *sv = slot_val + (size_t)sidx * W + lane_in * VEC;
+        } else {
+            const int slot = slot_of[u];
+            if (slot < 0) return;
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
+                const size_t o = (size_t)slot * C + col + k;
                 if constexpr (kMax) {
-                    sv[k] = idx[k] >= 0 ? (((unsigned long long)ordered_bits((float)acc[k]) << 32) |
-                                           (unsigned long long)(0xffffffffu - low_word(idx[k])))
-                                        : 0ull;
+                    if (ix[k] >= 0)
+                        atomicMax(scratch + o, ((unsigned long long)ordered_bits((float)a[k]) << 32) |
+                                                   (unsigned long long)(0xffffffffu - low_word(ix[k], u)));
                 } else {
-                    sv[k] = (double)acc[k];
-                }
-            }
-        }
-        else if constexpr (CHUNK > kChunk) {
-            // A third heavy partial in one chunk: only the long chunk can meet one, with a plan
-            // whose heavy threshold is below its length (the threshold is never below the
-            // short chunk).  It goes straight to the table.
-            const int slot = slot_of[u];
-            if (slot >= 0) {
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) {
-                    const size_t o = (size_t)slot * C + col + k;
-                    if constexpr (kMax) {
-                        if (idx[k] >= 0)
-                            atomicMax(scratch + o, ((unsigned long long)ordered_bits((float)acc[k]) << 32) |
-                                                       (unsigned long long)(0xffffffffu - low_word(idx[k])));
-                    } else {
-                        unsafeAtomicAdd(reinterpret_cast<float *>(scratch) + o, acc[k]);
-                    }
+                    unsafeAtomicAdd(reinterpret_cast<float *>(scratch) + o, (float)a[k]);
                 }
             }
         }
     };
 
-    // Fold one loaded row (position l, voxel sg) into the running reduction.  With
-    // kGate the row counts only when `valid` (a slot past the range in the last
-    // batch of a chunk); the loaded registers are consumed on a straight-line path
-    // either way so the compiler can count outstanding loads exactly.
-    auto add_row = [&](auto gate, const Pack<raw, VEC> &v, int sg, int row, int l, bool valid) {
-        constexpr bool kGate = decltype(gate)::value;
-        if ((!kGate || valid) && sg != cur) {
-            flush(l);
-            cur = sg;
-            run_l0 = l;
-            rel0 = rel_of_run_start(sg, l);
+    // Fold the reduction (b, bi) of EARLIER rows of the same voxel into (a, ix).
+    auto fold_earlier = [&](AccT(&a)[VEC], int(&ix)[VEC], const AccT(&b)[VEC], const int(&bi)[VEC], int u) {
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) {
-                acc[k] = acc0;
-                idx[k] = -1;
+        for (int k = 0; k < VEC; ++k) {
+            if constexpr (!kMax) {
+                a[k] += b[k];
+            } else {
+                bool take = b[k] > a[k];
+                if (bi[k] >= 0 && b[k] == a[k]) {
+                    // equal values: the earlier row wins, or the smaller tie key of the reference
+                    take = ix[k] < 0 || !kRef || ref_key_at(bi[k], u) < ref_key_at(ix[k], u);
+                }
+                if (take) {
+                    a[k] = b[k];
+                    ix[k] = bi[k];
+                }
             }
         }
-        const int tag = kRef ? l : row;
-        if constexpr (!kMax && !kGate && TXS_F16_FMA_MIX && std::is_same<TR, F16>::value && VEC % 2 == 0) {
+    };
+
+    // A run ends at position l.
+    auto on_end = [&](auto staged, int l) {
+        constexpr bool kStaged = decltype(staged)::value;
+        const int sgv = kStaged ? seg_s[l] : seg_at(l);
+        if (pend_head) {
+            pend_head = false;
+            head_seg = sgv;
+            head_l = l;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                hacc[k] = acc[k];
+                hidx[k] = idx[k];
+            }
+        } else {
+            emit(staged, sgv, acc, idx, l + 1 - run_l0, (long)t0 - 1 + run_l0, (long)t0 + l);
+        }
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            acc[k] = acc0;
+            idx[k] = -1;
+        }
+        run_l0 = l + 1;
+    };
+
+    // Fold one loaded row (position l, staged word pk) into the running reduction.
+    auto add_row = [&](auto staged, const Pack<raw, VEC> &v, int l, int pk) {
+        constexpr bool kStaged = decltype(staged)::value;
+        const int tag = kRef ? l : (pk & kIdMask);
+        if constexpr (!kMax && TXS_F16_FMA_MIX && std::is_same<TR, F16>::value && VEC % 2 == 0) {
             unsigned w[VEC / 2 > 0 ? VEC / 2 : 1];
             __builtin_memcpy(w, &v, sizeof(unsigned) * (VEC / 2));
 #pragma unroll
@@ -301,21 +362,22 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
         }
         if constexpr (kRef) {
             // Reference-tie mode also takes an equal value whose tie key is smaller.  Equal
-            // values are rare, so the keys (of this row's offset in its voxel and of the
-            // current winner's) are only worked out where a lane meets one.
+            // values are rare, so the keys are only worked out where a lane meets one.
             bool tie = false;
 #pragma unroll
             for (int k = 0; k < VEC; ++k) tie |= TR::to_m(v.v[k]) == acc[k];
-            if (kGate) tie &= valid;
             if (__builtin_expect(tie, 0)) {
-                const unsigned kn = (unsigned)ref_key(rel0 + (l - run_l0), ref_log2);
+                const int u = (kStaged ? seg_s[l] : seg_at(l)) & kIdMask;
+                if ((unsigned)u < (unsigned)U) {
+                    const unsigned kn = ref_key_at(l, u);
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) {
-                    if (!(TR::to_m(v.v[k]) == acc[k])) continue;
-                    const unsigned ko = idx[k] < 0 ? 0xffffffffu : (unsigned)ref_key(rel0 + (idx[k] - run_l0), ref_log2);
-                    if (kn < ko) {  // the value's bits follow the winner (a zero's sign)
-                        idx[k] = tag;
-                        acc[k] = TR::to_m(v.v[k]);
+                    for (int k = 0; k < VEC; ++k) {
+                        if (!(TR::to_m(v.v[k]) == acc[k])) continue;
+                        const unsigned ko = idx[k] < 0 ? 0xffffffffu : ref_key_at(idx[k], u);
+                        if (kn < ko) {  // the value's bits follow the winner (a zero's sign)
+                            idx[k] = tag;
+                            acc[k] = TR::to_m(v.v[k]);
+                        }
                     }
                 }
             }
@@ -325,155 +387,125 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
             if constexpr (kMax) {
                 const AccT x = TR::to_m(v.v[k]);
                 // strict '>': the first row wins ties, NaN never wins
-                bool take = x > acc[k];
-                if (kGate) take &= valid;
+                const bool take = x > acc[k];
                 acc[k] = take ? x : acc[k];
                 idx[k] = take ? tag : idx[k];
             } else {
-                const float x = TR::to_f(v.v[k]);
-                acc[k] += (!kGate || valid) ? x : 0.0f;
+                acc[k] += TR::to_f(v.v[k]);
             }
         }
     };
 
-    // Row r of the feature matrix at this lane's columns: one 64-bit multiply-add.
-    // A row index outside the matrix (only a corrupt plan has one) is clamped.
-    const char *lane_base = reinterpret_cast<const char *>(feats) + (size_t)col * sizeof(raw);
-    const unsigned row_bytes = (unsigned)C * (unsigned)sizeof(raw);
-    const unsigned last_row = (unsigned)(N - 1);
-    auto row_ptr = [&](int r) -> const raw * {
-        const unsigned rc = min((unsigned)r, last_row);
-        return reinterpret_cast<const raw *>(lane_base + (unsigned long long)rc * row_bytes);
-    };
-
-    // Every slot of a batch issues a load (slots past the range re-load the
-    // range's last row, a cache hit) so that no load sits under a branch.
-    // A batch keeps only the loaded rows; the voxel and row ids are read again from LDS
-    // when the batch is reduced (fewer live registers: one more wave per SIMD for sum/mean).
-    struct Batch {
-        Pack<raw, VEC> v[kBatch];
-    };
-    auto issue = [&](Batch &bt, int l) {
+    if (live) {
+        // Every lane group walks `ch` steps (the last one empty for those with a row less), so
+        // the lane groups of a wavefront stay in step.  Row loads are double-buffered, every
+        // load is issued on a straight-line path (slots past the share re-load its last row, a
+        // cache hit) and the prefetch loop is peeled, so that the counts of loads in flight
+        // are known where a batch is reduced.
+        struct Batch {
+            Pack<raw, VEC> v[kBatch];
+        };
+        const int l_stop = c0 + ch;  // the same distance for every lane group
+        const int l_clamp = max(c_end - 1, c0);
+        auto issue = [&](Batch &bt, int l) {
 #pragma unroll
-        for (int i = 0; i < kBatch; ++i) {
-            const int lc = min(l + i, lb_fast - 1);
-            bt.v[i] = ld_stream<raw, VEC>(row_ptr(perm_s[lc - 1]));
-        }
-    };
-    // A batch that lies wholly inside the range needs no per-row gate; only the
-    // last batch of a chunk can hold slots past the range.
-    auto consume_full = [&](const Batch &bt, int l) {
+            for (int i = 0; i < kBatch; ++i) bt.v[i] = ld_stream<raw, VEC>(row_ptr(pk_s[min(l + i, l_clamp) - 1] & kIdMask));
+        };
+        auto consume_full = [&](const Batch &bt, int l) {
 #pragma unroll
-        for (int i = 0; i < kBatch; ++i)
-            add_row(std::false_type{}, bt.v[i], seg_s[l + i], perm_s[l + i - 1], l + i, true);
-    };
-    auto consume_last = [&](const Batch &bt, int l) {
+            for (int i = 0; i < kBatch; ++i) {
+                const int pk = pk_s[l + i - 1];
+                add_row(std::true_type{}, bt.v[i], l + i, pk);
+                if (pk < 0) on_end(std::true_type{}, l + i);
+            }
+        };
+        auto consume_last = [&](const Batch &bt, int l) {
 #pragma unroll
-        for (int i = 0; i < kBatch; ++i) {
-            const int lc = min(l + i, lb_fast - 1);
-            add_row(std::true_type{}, bt.v[i], seg_s[lc], perm_s[lc - 1], l + i, l + i < lb_fast);
+            for (int i = 0; i < kBatch; ++i) {
+                if (l + i < c_end) {
+                    const int pk = pk_s[l + i - 1];
+                    add_row(std::true_type{}, bt.v[i], l + i, pk);
+                    if (pk < 0) on_end(std::true_type{}, l + i);
+                }
+            }
+        };
+        Batch b0, b1;
+        issue(b0, c0);
+        for (int l = c0;;) {
+            int ln = l + kBatch;
+            if (ln >= l_stop) {
+                consume_last(b0, l);
+                break;
+            }
+            issue(b1, ln);
+            consume_full(b0, l);
+            l = ln;
+            ln = l + kBatch;
+            if (ln >= l_stop) {
+                consume_last(b1, l);
+                break;
+            }
+            issue(b0, ln);
+            consume_full(b1, l);
+            l = ln;
         }
-    };
-
-    // Positions staged in LDS go through the double-buffered loop; the rare rest
-    // (an ordinary run longer than kMargin crossing the tile's end) is walked
-    // one row at a time with its ids fetched from global memory.
-    // Each prefetch is unconditional on its path, so the count of loads in
-    // flight is known at every use: a batch is reduced while the next one is
-    // still arriving.
-    Batch b0, b1;
-    issue(b0, la);
-    for (int l = la;;) {
-        int ln = l + kBatch;
-        if (ln >= lb_fast) {
-            consume_last(b0, l);
-            break;
-        }
-        issue(b1, ln);
-        consume_full(b0, l);
-        l = ln;
-        ln = l + kBatch;
-        if (ln >= lb_fast) {
-            consume_last(b1, l);
-            break;
-        }
-        issue(b0, ln);
-        consume_full(b1, l);
-        l = ln;
-    }
-    for (int l = lb_fast; l < lb; ++l) {
-        const int r = row_at(l);
-        if ((unsigned)r >= (unsigned)N) continue;
-        add_row(std::false_type{}, ld_stream<raw, VEC>(row_ptr(r)), seg_at(l), r, l, true);
-    }
-    flush(lb);
-    };  // reduce_chunk
-    reduce_chunk();
-
-    // Workgroup-level merge of the parked partials.  The used slots that carry
-    // the same voxel id form one range (a heavy run is contiguous in sorted
-    // order, so only unused slots can sit between them).  All 256 threads take
-    // part: (A) mark the first slot of every range, (B) fold every other slot
-    // into its range's first slot with LDS atomics, (C) send each range total to
-    // the global table with one atomic per element.  Tiles without a heavy voxel
-    // skip all of this and its barriers.
-    if (!tile_has_heavy) return;
-    __shared__ unsigned long long start_mask[(2 * kThreads) / 64];
-    const int S = 2 * G;                       // slots in this workgroup
-    const int w_log2 = lpr_log2 + (VEC == 8 ? 3 : VEC == 4 ? 2 : VEC == 2 ? 1 : 0);  // log2(W)
-    __syncthreads();
-    for (int base = 0; base < S; base += kThreads) {
-        const int sl = base + (int)threadIdx.x;
-        bool first = false;
-        if (sl < S) {
-            const int id = slot_id[sl];
-            if (id >= 0) {
-                int prev = sl - 1;
-                while (prev >= 0 && slot_id[prev] < 0) --prev;
-                first = prev < 0 || slot_id[prev] != id;
+        if (c0 < c_end) {
+            const int l_last = c_end - 1;
+            const int sg_last = seg_s[l_last];
+            const bool open = pk_s[l_last - 1] >= 0 && sg_last != kNoSeg;
+            if (open && c_end == b_hi) {
+                if (sg_last >= 0 && long_tail) {
+                    // (rare) the range ends inside an ordinary run whose end lies beyond the
+                    // staged ids: walk on to it
+                    for (int l = c_end;; ++l) {
+                        const int pk = pk_at(l);
+                        if (seg_at(l) == kNoSeg) break;
+                        add_row(std::false_type{}, ld_stream<raw, VEC>(row_ptr(pk & kIdMask)), l, pk);
+                        if (pk < 0) {
+                            on_end(std::false_type{}, l);
+                            break;
+                        }
+                    }
+                } else if (sg_last < 0) {
+                    // the range ends inside a heavy run: its rows in this tile are complete here
+                    on_end(std::true_type{}, l_last);
+                }
+            } else if (open) {
+                float *cv = carry_v + (size_t)threadIdx.x * VEC;
+                int *ci = carry_i + (size_t)threadIdx.x * VEC;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    cv[k] = (float)acc[k];
+                    if (kMax) ci[k] = idx[k];
+                }
             }
         }
-        const unsigned long long m = __ballot(first);
-        if ((threadIdx.x & 63) == 0) start_mask[(base + (int)threadIdx.x) >> 6] = m;
     }
     __syncthreads();
-    // first slot of the range that slot sl belongs to: nearest marked slot at or below sl
-    auto range_start = [&](int sl) -> int {
-        int wd = sl >> 6;
-        unsigned long long m = start_mask[wd] & (~0ull >> (63 - (sl & 63)));
-        while (m == 0ull && wd > 0) m = start_mask[--wd];
-        return m ? (wd << 6) + 63 - __builtin_clzll(m) : sl;
-    };
-    for (int i = threadIdx.x; i < (S << w_log2); i += kThreads) {
-        const int sl = i >> w_log2, e = i & (W - 1);
-        if (slot_id[sl] < 0) continue;
-        const int head = range_start(sl);
-        if (head == sl) continue;
-        const SlotT x = slot_val[i];
-        SlotT *dst = slot_val + ((size_t)head << w_log2) + e;
-        if constexpr (kMax) {
-            if (x != 0ull) atomicMax(dst, x);
-        } else {
-            __hip_atomic_fetch_add(dst, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (!live || head_seg == kNoSeg) return;
+    // The kept head: add what the lane groups before this one reduced of the same run (a
+    // heavy run can cover many shares), then write it out.  An ordinary run always starts inside
+    // the tile's range; a heavy one that began in an earlier tile leaves its rows of this tile.
+    int first_l = c0;
+    for (int k = gi - 1; k >= 0; --k) {
+        const int k0 = share_begin(k);
+        if (k0 == share_begin(k + 1)) continue;  // a lane group without rows
+        const float *cv = carry_v + ((size_t)(k << lpr_log2) + lane_in) * VEC;
+        const int *ci = carry_i + ((size_t)(k << lpr_log2) + lane_in) * VEC;
+        AccT b[VEC];
+        int bi[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            b[e] = (AccT)cv[e];
+            bi[e] = kMax ? ci[e] : 0;
         }
+        fold_earlier(hacc, hidx, b, bi, head_seg & kIdMask);
+        first_l = k0;
+        if (seg_s[k0 - 1] != head_seg) break;  // the run starts in this share
     }
-    __syncthreads();
-    for (int i = threadIdx.x; i < (S << w_log2); i += kThreads) {
-        const int sl = i >> w_log2, e = i & (W - 1);
-        if (!((start_mask[sl >> 6] >> (sl & 63)) & 1ull)) continue;
-        const int c = (((int)blockIdx.y << lpr_log2) * VEC) + e;
-        if (c >= C) continue;
-        const int id = slot_id[sl];
-        const int slot = ((unsigned)id < (unsigned)U) ? slot_of[id] : -1;
-        if (slot < 0) continue;
-        const SlotT tot = slot_val[i];
-        const size_t o = (size_t)slot * C + c;
-        if constexpr (kMax) {
-            if (tot != 0ull) atomicMax(scratch + o, tot);
-        } else {
-            unsafeAtomicAdd(reinterpret_cast<float *>(scratch) + o, (float)tot);
-        }
-    }
+    const int u = head_seg & kIdMask;
+    const int cnt = ((unsigned)u < (unsigned)U && head_seg >= 0) ? preSum[u + 1] - preSum[u] : 1;
+    emit(std::false_type{}, head_seg, hacc, hidx, cnt, (long)t0 - 1 + first_l, (long)t0 + head_l);
 }
 
 // Turn the scratch table of the special voxels into output rows and clear it.
@@ -695,8 +727,8 @@ Geometry make_geometry(long N, long C, int elem, const void *p0, const void *p1,
     const long tile = (long)(kThreads >> l2) * chunk;  // sorted positions per workgroup
     long blocks = (N + tile - 1) / tile;
     blocks = (blocks + 8 * kXcdSpan - 1) / (8 * kXcdSpan) * (8 * kXcdSpan);
-    g.lds_fwd_idx = (unsigned)((((2 * (tile + kMargin) + 1) + 2 * (kThreads >> l2) + 1) & ~1L) * sizeof(int));
-    g.lds_slots = (unsigned)(2 * kThreads * vec);
+    g.lds_fwd_idx = (unsigned)(((2 * (tile + kMargin + 1) + 1 + 3) & ~3L) * sizeof(int));
+    g.lds_slots = (unsigned)(2 * kThreads * vec);  // carry cells: a value and a tag per element
     g.lds_bwd = (unsigned)(2 * tile * sizeof(int));
     g.grid = dim3((unsigned)blocks, (unsigned)g.ytiles, 1);
     return g;
@@ -711,7 +743,7 @@ hipError_t launch_fwd_op(int op, const Geometry &geo, hipStream_t st, const void
     auto o = (raw *)out;
     auto s = (unsigned long long *)scratch;
     dim3 blk(kThreads);
-    const unsigned lds8 = geo.lds_fwd_idx + 8 * geo.lds_slots;  // 8-byte slot cells for every operator
+    const unsigned lds8 = geo.lds_fwd_idx + 4 * geo.lds_slots;  // staged ids, then 4-byte carry cells
 #define TXS_FWD_OP(OPC)                                                                           \
     if (geo.chunk == kChunkLong)                                                                  \
         scatter_fwd_kernel<TR, VEC, OPC, kChunkLong><<<geo.grid, blk, lds8, st>>>(                \

@@ -46,6 +46,9 @@ namespace {
 #ifndef TXS_BATCH_HALF_MAX
 #define TXS_BATCH_HALF_MAX 6
 #endif
+#ifndef TXS_FAST_DIV_HALF
+#define TXS_FAST_DIV_HALF 1
+#endif
 #ifndef TXS_NT_LOADS
 #define TXS_NT_LOADS 1
 #endif
