@@ -1,24 +1,26 @@
 // Voxel scatter-reduction kernels for MI355X (gfx950, wave64) and their C ABI.
 //
 // Design in one paragraph.  Index preparation sorts row ids by voxel id once
-// (stable LSD radix sort) and stores, for every sorted position j, the row
-// perm[j] and the voxel seg[j].  The forward pass is then a segmented reduction
-// over sorted positions: a "lane group" (the lanes that together cover one
-// feature row, each lane owning one 128-bit channel vector) walks a fixed-size
-// chunk of positions, keeps the running sum / max of the current voxel in
+// and stores, for every sorted position j, the row perm[j] and the voxel seg[j].
+// The forward pass is then a segmented reduction over sorted positions: a "lane
+// group" (the lanes that together cover one feature row, each lane owning one
+// 128-bit channel vector) keeps the running sum / max of the current voxel in
 // registers and writes a voxel's output row exactly once when its run of equal
-// ids ends.  A run that starts in a chunk is finished by the same lane group
-// even if it spills into the next chunk, so ordinary voxels never need an
-// atomic.  Only voxels above the heavy threshold are split across lane groups;
-// their per-chunk partials are first merged inside the workgroup through LDS,
-// then meet in a scratch table through fp32 atomic adds (sum/mean) or a 64-bit
-// atomic max on a packed (ordered value | ~row) word (max/argmax), and a small
-// finalize kernel turns the table into output rows.  The backward pass is a
-// gather over the same sorted positions: the upstream row of a voxel is read
-// once per run and every row of the input gradient is written exactly once,
-// with no zero-fill pass and no atomics.  The same sort also serves the callers
-// on either side of the path: voxel keys from points, the unique/inverse/counts
-// triple, and the rank of a point inside its voxel.
+// ids ends.  A workgroup owns a tile of positions whose borders are moved to the
+// next run start, so that an ordinary voxel lies in one tile, and deals the tile's
+// rows evenly to its lane groups: all lane groups of a wavefront walk the same
+// number of rows.  A run that crosses the border between two lane groups is
+// completed after one barrier: the earlier group leaves its part in LDS, the group
+// that holds the run's end adds it.  Only voxels above the heavy threshold are
+// split across tiles; their per-tile partials meet in a scratch table through one
+// fp32 atomic add (sum/mean) or one 64-bit atomic max on a packed (ordered value |
+// ~row) word (max/argmax) per element and tile, and a small finalize kernel turns
+// the table into output rows.  The backward pass is a gather over the same sorted
+// positions: the upstream row of a voxel is read once per run and every row of the
+// input gradient is written exactly once, with no zero-fill pass and no atomics.
+// The same sort also serves the callers on either side of the path: voxel keys
+// from points, the unique/inverse/counts triple, and the rank of a point inside
+// its voxel.
 //
 // Reference behaviour being replaced: torchex/src/scatter/scatter_kernel.cu
 // (getPreSum :85-100, scatter_sum :102-129, scatter_max :131-171) and the
@@ -44,13 +46,18 @@ namespace {
 
 // ----------------------------------------------------------------- forward --
 //
-// One workgroup owns a tile of G * kChunk consecutive sorted positions, where
-// G = 256 / (lanes per row) lane groups each own kChunk of them.  The tile's seg
-// and perm entries (plus one entry before and kMargin after) are staged in LDS
-// by one coalesced load, so the row loads that follow never wait on an index
-// load, and a lane group can look across its chunk borders for free.  Row loads
-// are double-buffered: the next batch is in flight while the current one is
-// reduced.
+// One workgroup owns a tile of G * chunk consecutive sorted positions (G = 256 /
+// (lanes per row) lane groups).  The tile's seg and perm entries (plus one entry
+// before and kMargin after) are staged in LDS by one coalesced load, so the row
+// loads that follow never wait on an index load.  The tile's own range runs from
+// the first run start at or after its first position to the first run start at or
+// after the next tile's first position (a heavy run is cut anywhere): it is dealt
+// to the lane groups in shares that differ by one row at most.  Measured on the
+// LiDAR sweep before this: chunks of a fixed 16 positions whose owner skipped the
+// tail of a run begun earlier and finished the run open at its end gave the lane
+// groups 16 +- 9.7 rows, and a wavefront walked 39 % more rows than it reduced.
+// Row loads are double-buffered: the next batch is in flight while the current one
+// is reduced.
 
 constexpr int kMargin = 64;           // staged entries past the tile's end
 constexpr int kNoSeg = 0x7fffffff;    // never a valid seg value
@@ -79,24 +86,26 @@ __device__ __forceinline__ int ref_rel(int key, int blog2) {  // inverse of ref_
     return (int)((iter << blog2) | ref_prio((unsigned)key >> kIterBits, blog2 - 5));
 }
 
-template <class TR, int VEC, int OP, int CHUNK>
+template <class TR, int VEC, int OP>
 __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     const typename TR::raw *__restrict__ feats, const int *__restrict__ perm,
     const int *__restrict__ seg, const int *__restrict__ slot_of,
     typename TR::raw *__restrict__ out, int *__restrict__ arg,
     unsigned long long *__restrict__ scratch, const int *__restrict__ preSum, int N, int C, int U,
-    int lpr_log2, int ref_log2) {
+    int lpr_log2, int ref_log2, int chunk) {
     using raw = typename TR::raw;
     constexpr bool kMax = OP == TXS_MAX || OP == TXS_MAX_REFTIE;
     constexpr bool kRef = OP == TXS_MAX_REFTIE;  // idx[] then holds the winner's staged position, not its row
-    // (the fp16 running max keeps packed halves and has registers to spare for a deeper batch)
-    constexpr int kBatch = sizeof(raw) == 2 ? ((kMax && std::is_same<TR, F16>::value) ? kBatchHalfMax : kBatchHalf) : ::kBatch;
+    // rows per load batch (two batches in flight); measured per dtype and operator
+    constexpr int kBatch = sizeof(raw) == 2
+                               ? (kMax ? (std::is_same<TR, F16>::value ? kBatchHalfMax : kBatchBf16Max) : kBatchHalf)
+                               : ::kBatch;
     using AccT = typename std::conditional<kMax, typename TR::max_t, float>::type;
     constexpr int kEndBit = kSpecialBit;
     extern __shared__ int lds[];
     const int g_log2 = 8 - lpr_log2;      // kThreads == 256
     const int G = 1 << g_log2;
-    const int T = G * CHUNK;
+    const int T = G * chunk;              // `chunk` positions per lane group on average
     const int n_seg_s = T + kMargin + 1;  // positions t0-1 .. t0+T+kMargin-1
     int *seg_s = lds;                     // seg_s[l]: voxel (bit 31: special) at position t0 - 1 + l
     int *pk_s = lds + n_seg_s;            // pk_s[l - 1]: row at position t0 - 1 + l, bit 31 = last row of its run
@@ -682,14 +691,18 @@ __global__ __launch_bounds__(kThreads) void scatter_bwd_kernel(
 
 // ------------------------------------------------------------------ launch --
 
-// Sorted positions per lane group of the forward kernel: the long chunk when runs are long on
-// average (fewer heavy-voxel partials to park and merge per row), the short one otherwise
-// (shorter dependent walks, more workgroups).  Between 8 and 64 rows per voxel the long chunk
-// pays for max and for the 2-byte types, whose merges weigh more against their row work; the
-// fp32 sum / mean kernels and the reference-tie max are faster with the short one there.
+// Sorted positions per lane group of the forward kernel (on average: a tile's range is dealt
+// evenly).  Long runs (64 rows per voxel and more) are reduced fastest in tiles of 32 positions
+// per lane group (fewer tile borders for a run to cross, one atomic row per tile and heavy
+// voxel); short runs of 4-byte elements in tiles of 8 (twice the workgroups, shorter dependent
+// walks: 4 % on the LiDAR sweep, 8 % on 200k rows); everything else in tiles of 16.
 int fwd_chunk_for(long N, long U, int op, int elem) {
+#ifdef TXS_FORCE_FWD_CHUNK
+    return TXS_FORCE_FWD_CHUNK;
+#endif
+    (void)op;
     if (N >= 64 * U) return kChunkLong;
-    return (N >= 8 * U && op != TXS_MAX_REFTIE && (op == TXS_MAX || elem == 2)) ? kChunkLong : kChunk;
+    return (elem == 4 && N < 8 * U) ? kChunkShort : kChunk;
 }
 
 struct Geometry {
@@ -704,7 +717,7 @@ struct Geometry {
 bool aligned_to(const void *p, int bytes) { return p == nullptr || ((uintptr_t)p % (uintptr_t)bytes) == 0; }
 
 Geometry make_geometry(long N, long C, int elem, const void *p0, const void *p1, const void *p2,
-                       bool arg_used, const void *parg, int chunk) {
+                       bool arg_used, const void *parg, int chunk, bool forward = false) {
     Geometry g;
     // bytes per lane and row: 16 for fp32; 8 for the 2-byte types, whose kernels carry
     // twice the registers per byte (measured 4-12 % faster than 16 on fp16 / bf16)
@@ -717,12 +730,15 @@ Geometry make_geometry(long N, long C, int elem, const void *p0, const void *p1,
         vb >>= 1;
     }
     g.vec_bytes = vb;
-    g.chunk = chunk;
     const long vec = vb / elem;
     const long lanes = (C + vec - 1) / vec;
     int l2 = 0;
     while ((1L << l2) < lanes && l2 < 6) ++l2;
     g.lpr_log2 = l2;
+    // a tile (lane groups x chunk positions) is a whole number of wavefronts' worth of staged
+    // ids: the forward kernel finds the borders of a tile's range with one ballot each
+    while (forward && ((long)(kThreads >> l2) * chunk) % 64 != 0) chunk *= 2;
+    g.chunk = chunk;
     g.ytiles = (int)((lanes + (1L << l2) - 1) >> l2);
     const long tile = (long)(kThreads >> l2) * chunk;  // sorted positions per workgroup
     long blocks = (N + tile - 1) / tile;
@@ -744,13 +760,9 @@ hipError_t launch_fwd_op(int op, const Geometry &geo, hipStream_t st, const void
     auto s = (unsigned long long *)scratch;
     dim3 blk(kThreads);
     const unsigned lds8 = geo.lds_fwd_idx + 4 * geo.lds_slots;  // staged ids, then 4-byte carry cells
-#define TXS_FWD_OP(OPC)                                                                           \
-    if (geo.chunk == kChunkLong)                                                                  \
-        scatter_fwd_kernel<TR, VEC, OPC, kChunkLong><<<geo.grid, blk, lds8, st>>>(                \
-            f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);           \
-    else                                                                                          \
-        scatter_fwd_kernel<TR, VEC, OPC, kChunk><<<geo.grid, blk, lds8, st>>>(                    \
-            f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2);
+#define TXS_FWD_OP(OPC)                                                            \
+    scatter_fwd_kernel<TR, VEC, OPC><<<geo.grid, blk, lds8, st>>>(                 \
+        f, perm, seg, slot_of, o, arg, s, preSum, N, C, U, geo.lpr_log2, ref_log2, geo.chunk);
     switch (op) {
         case TXS_SUM: TXS_FWD_OP(TXS_SUM) break;
         case TXS_MEAN: TXS_FWD_OP(TXS_MEAN) break;
@@ -939,7 +951,7 @@ int scatter_forward_impl(int op, int dtype, const void *feats, const int32_t *un
         if (hipGetLastError() != hipSuccess) return TXS_ERR_LAUNCH;
     }
     if (N > 0) {
-        Geometry geo = make_geometry(N, C, elem, feats, out, nullptr, is_max, arg, fwd_chunk_for(N, U, op, elem));
+        Geometry geo = make_geometry(N, C, elem, feats, out, nullptr, is_max, arg, fwd_chunk_for(N, U, op, elem), true);
         if (dtype == TXS_F32)
             e = launch_fwd<F32>(op, geo, st, feats, perm, seg, preSum, slot_of, out, arg, scratch, N, C, U, ref_log2);
         else if (dtype == TXS_F16)
@@ -1009,9 +1021,8 @@ int txs_kernel_name(int backward, int op, int dtype, int64_t num_total, int64_t 
     } else {
         const bool is_max = op == TXS_MAX || op == TXS_MAX_REFTIE;
         const Geometry geo = make_geometry(num_total, channel, elem, p, p, nullptr, is_max, p,
-                                           fwd_chunk_for(num_total, num_unq, op, elem));
-        snprintf(buf, (size_t)buf_len, "scatter_fwd_kernel<%s,%d,%s,%d>", kTypes[dtype], geo.vec_bytes / elem,
-                 kOps[op], geo.chunk);
+                                           fwd_chunk_for(num_total, num_unq, op, elem), true);
+        snprintf(buf, (size_t)buf_len, "scatter_fwd_kernel<%s,%d,%s>", kTypes[dtype], geo.vec_bytes / elem, kOps[op]);
     }
     return TXS_OK;
 }

@@ -44,7 +44,10 @@ namespace {
 #define TXS_F16_FMA_MIX 1
 #endif
 #ifndef TXS_BATCH_HALF_MAX
-#define TXS_BATCH_HALF_MAX 6
+#define TXS_BATCH_HALF_MAX 4
+#endif
+#ifndef TXS_BATCH_BF16_MAX
+#define TXS_BATCH_BF16_MAX 8
 #endif
 #ifndef TXS_FAST_DIV_HALF
 #define TXS_FAST_DIV_HALF 1
@@ -59,6 +62,7 @@ namespace {
 constexpr int kThreads = 256;        // 4 wavefronts per workgroup
 constexpr int kChunk = TXS_CHUNK;    // sorted positions per lane group (forward)
 constexpr int kChunkLong = 2 * TXS_CHUNK;  // the same when runs are long on average
+constexpr int kChunkShort = TXS_CHUNK / 2;  // ... and for short runs of 4-byte elements
 constexpr int kChunkBwdShort = TXS_CHUNK_BWD_SHORT;  // backward kernel, mean run shorter than kChunkBwdLong
 constexpr int kChunkBwdLong = TXS_CHUNK;             // backward kernel, longer runs
 constexpr int kBatchBwd = TXS_BATCH_BWD;
@@ -66,6 +70,7 @@ constexpr int kBatch = TXS_BATCH;    // rows per load batch of a lane group (two
 constexpr int kBatchHalf = TXS_BATCH_HALF;         // the same for the 2-byte types
 constexpr int kBatchBwdHalf = TXS_BATCH_BWD_HALF;
 constexpr int kBatchHalfMax = TXS_BATCH_HALF_MAX;  // forward max of fp16
+constexpr int kBatchBf16Max = TXS_BATCH_BF16_MAX;  // forward max of bf16
 constexpr int kHalfVecBytes = TXS_HALF_VEC_BYTES;  // bytes one lane moves per row for fp16 / bf16
 constexpr int kHeavyDefault = 64;    // voxels above this many rows use the atomic path
 constexpr int kTableMinRowsPerVoxel = 512;  // table mode needs at least this many rows per voxel on average
