@@ -86,14 +86,14 @@ def test_argument_validation_needs_no_gpu():
     buf = ctypes.create_string_buffer(64)
     assert lib.txs_kernel_name(ci(0), ci(2), ci(0), i64(1_000_000), i64(128), i64(300_000), i64(16), ci(1), buf,
                                i64(64)) == 0
-    assert buf.value == b"scatter_fwd_kernel<F32,4,MAX,16>"
+    assert buf.value == b"scatter_fwd_kernel<F32,4,MAX>"
     assert lib.txs_kernel_name(ci(1), ci(1), ci(1), i64(1_000_000), i64(128), i64(300_000), i64(16), ci(1), buf,
                                i64(64)) == 0
     assert buf.value == b"scatter_bwd_kernel<F16,4,MEAN,8>"
     # long runs on average: the forward walks longer chunks
     assert lib.txs_kernel_name(ci(0), ci(0), ci(1), i64(1_000_000), i64(128), i64(89_260), i64(16), ci(1), buf,
                                i64(64)) == 0
-    assert buf.value == b"scatter_fwd_kernel<F16,4,SUM,32>"
+    assert buf.value == b"scatter_fwd_kernel<F16,4,SUM>"
     rc = lib.txs_get_presum(vp(0), vp(0), i64(-1), i64(0), vp(0))
     assert rc == 1
     # the unique-by-occupancy-map and ranking entry points: sizes and null pointers are checked first
