@@ -314,6 +314,33 @@ def test_heavy_runs_shorter_than_the_long_chunk(C):
     run_case("short_heavy_runs_f16", feats, inv_sorted[p], cnts, heavy_threshold=16, dtype=torch.float16)
 
 
+@pytest.mark.parametrize("C,dtype", [(16, torch.float32), (128, torch.float32), (128, torch.float16), (3, torch.float32)])
+def test_ordinary_runs_longer_than_a_tile(C, dtype):
+    """A heavy threshold far above the run lengths: every voxel is reduced in registers, also
+    those whose runs are longer than the ids a tile stages behind its end (64) and longer than
+    whole tiles.  A tile then finds no run start behind its end and its last lane group walks on
+    to the run's end; a tile that lies inside such a run finds none behind its start either and
+    owns nothing; runs of a few rows sit between the long ones."""
+    g = torch.Generator().manual_seed(77)
+    sizes = []
+    for _ in range(120):
+        sizes += [int(torch.randint(65, 700, (1,), generator=g)), int(torch.randint(1, 9, (1,), generator=g)),
+                  int(torch.randint(1, 4, (1,), generator=g))]
+    sizes += [2500, 1, 64, 65, 129, 1, 1, 300]
+    cnts = torch.tensor(sizes, dtype=torch.long)
+    U = len(sizes)
+    inv_sorted = torch.repeat_interleave(torch.arange(U), cnts)
+    N = int(cnts.sum())
+    feats = torch.randn((N, C), generator=g)
+    feats[torch.rand((N, C), generator=g) < 0.05] = 2.0          # ties
+    data = run_case("long_ordinary_runs_sorted", feats, inv_sorted, cnts, dtype=dtype, heavy_threshold=4000)
+    assert data.num_heavy == 0
+    p = torch.randperm(N, generator=g)
+    run_case("long_ordinary_runs_shuffled", feats, inv_sorted[p], cnts, dtype=dtype, heavy_threshold=4000)
+    run_case("long_ordinary_runs_first_tie", feats, inv_sorted, cnts, dtype=dtype, heavy_threshold=4000,
+             max_tie_rule="first")
+
+
 # ------------------------------------------------- the reference's own test --
 
 def test_reference_test_data_closed_forms(reference_counts):
