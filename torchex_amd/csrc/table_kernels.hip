@@ -35,7 +35,13 @@ constexpr int kTableLdsBudget = 144 * 1024;  // bytes of LDS a table may take (1
 #ifndef TXS_TABLE_UNROLL
 #define TXS_TABLE_UNROLL 2
 #endif
-constexpr int kTableUnroll = TXS_TABLE_UNROLL;  // rows per lane in flight
+#ifndef TXS_TABLE_HALF_SUM_VB
+#define TXS_TABLE_HALF_SUM_VB 4
+#endif
+#ifndef TXS_TABLE_MAX_PREFILTER
+#define TXS_TABLE_MAX_PREFILTER 1
+#endif
+constexpr int kTableUnroll = TXS_TABLE_UNROLL;  // rows per lane in flight (twice as many for lanes of 4 bytes or less in the forward)
 constexpr int kReduceThreads = 1024;
 constexpr int kReduceSplit = 64;             // lanes that share the partials of one output cell
 constexpr int kReduceLoads = 4;              // partials each of them has in flight
@@ -56,6 +62,7 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
     void *__restrict__ partials, int N, int C, int U, int lpr_log2, int stride, int rows_per_wg) {
     using raw = typename TR::raw;
     constexpr bool kMax = OP == TXS_MAX;
+    constexpr int kRows = sizeof(raw) * VEC <= 4 ? 2 * kTableUnroll : kTableUnroll;  // rows per lane in flight
     extern __shared__ unsigned long long table_lds[];
     unsigned long long *tkey = table_lds;
     double *tsum = reinterpret_cast<double *>(table_lds);
@@ -70,16 +77,16 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
     const long r0 = (long)blockIdx.x * rows_per_wg;
     const int r_end = (int)min((long)N, r0 + rows_per_wg);
     if (col < C) {
-        // Two batches of kTableUnroll rows per lane: the next one is on its way from memory
+        // Two batches of kRows rows per lane: the next one is on its way from memory
         // while the current one goes into the table.
         struct Batch {
-            int u[kTableUnroll];
-            Pack<raw, VEC> v[kTableUnroll];
+            int u[kRows];
+            Pack<raw, VEC> v[kRows];
         };
-        const int step = G * kTableUnroll;
+        const int step = G * kRows;
         auto issue = [&](Batch &b, int rb) {
 #pragma unroll
-            for (int k = 0; k < kTableUnroll; ++k) {
+            for (int k = 0; k < kRows; ++k) {
                 const int r = min(rb + k * G, r_end - 1);  // slots past the span re-load its last row
                 b.u[k] = inv[r] & kIdMask;
                 b.v[k] = TXS_TABLE_NT_LOADS ? ld_stream<raw, VEC>(feats + (size_t)r * C + col) : ld<raw, VEC>(feats + (size_t)r * C + col);
@@ -87,7 +94,7 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
         };
         auto consume = [&](const Batch &b, int rb) {
 #pragma unroll
-            for (int k = 0; k < kTableUnroll; ++k) {
+            for (int k = 0; k < kRows; ++k) {
                 const int r = rb + k * G;
                 if (r >= r_end || (unsigned)b.u[k] >= (unsigned)U) continue;
                 const int cell = b.u[k] * stride + col;
@@ -95,11 +102,16 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
                 for (int e = 0; e < VEC; ++e) {
                     const float x = TR::to_f(b.v[k].v[e]);
                     if constexpr (kMax) {
-                        if (x == x)  // NaN never wins
-                            __hip_atomic_fetch_max(tkey + cell + e,
-                                                   ((unsigned long long)ordered_bits(x) << 32) |
-                                                       (unsigned long long)(0xffffffffu - (unsigned)r),
-                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        // A cell only ever grows, so a key that does not beat a plain (possibly
+                        // stale) read of it cannot change it: after a voxel's first few rows
+                        // almost every row stops at the read, which costs a fraction of the atomic.
+                        const unsigned long long key = ((unsigned long long)ordered_bits(x) << 32) |
+                                                       (unsigned long long)(0xffffffffu - (unsigned)r);
+                        const bool beats = !(TXS_TABLE_MAX_PREFILTER && sizeof(raw) == 2) ||
+                            key > __hip_atomic_load(tkey + cell + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        if (x == x && beats)  // NaN never wins
+                            __hip_atomic_fetch_max(tkey + cell + e, key, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_WORKGROUP);
                     } else {
                         __hip_atomic_fetch_add(tsum + cell + e, (double)x, __ATOMIC_RELAXED,
                                                __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -426,7 +438,13 @@ TablePlan table_plan(bool backward, int op, int dtype, long N, long C, long U, l
     // few voxels, many rows each: a partial table per workgroup must stay small next to its rows
     if (N < (long)kTableMinRowsPerVoxel * U || N < 16384) return tp;
     const int elem = dtype == TXS_F32 ? 4 : 2;
-    const int vb = table_vec_bytes(C, elem, align);
+    int vb = table_vec_bytes(C, elem, align);
+    // 2-byte sum / mean: 4-byte lanes.  Wide lanes put many rows into one LDS atomic instruction,
+    // and rows of one voxel in the same instruction are served one after the other (2M rows of
+    // 16 channels into 1024 Zipf-distributed voxels: 42 us with 16-byte lanes, 35 with 8, 29
+    // with 4); fp32 rows, which take twice as long to stream, gain nothing from narrower lanes.
+    if (!backward && op != TXS_MAX && elem == 2)
+        while (vb > TXS_TABLE_HALF_SUM_VB && C * elem / (vb / 2) <= 64) vb /= 2;
     const int vec = vb / elem;
     const long lanes = (C + vec - 1) / vec;
     if (lanes > 64) return tp;
