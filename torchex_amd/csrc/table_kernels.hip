@@ -43,7 +43,7 @@ constexpr int kTableLdsBudget = 144 * 1024;  // bytes of LDS a table may take (1
 #endif
 constexpr int kTableUnroll = TXS_TABLE_UNROLL;  // rows per lane in flight (twice as many for lanes of 4 bytes or less in the forward)
 constexpr int kReduceThreads = 1024;
-constexpr int kReduceSplit = 64;             // lanes that share the partials of one output cell
+constexpr int kReduceSplit = 32;             // lanes that share the partials of one output cell
 constexpr int kReduceLoads = 4;              // partials each of them has in flight
 
 // ------------------------------------------------------------------ forward --
@@ -53,8 +53,8 @@ constexpr int kReduceLoads = 4;              // partials each of them has in fli
 // part an LDS fp32 atomic add retires about one lane every three cycles, whatever the
 // addresses, while fp64 and integer LDS atomics run seven times faster (2M rows of 16
 // channels into 1024 voxels: 164 us with fp32 cells, 26 us with fp64 cells, 20 us for the
-// load stream alone).  A workgroup's partial is stored as fp32 (sum / mean) or as the
-// packed word (max).
+// load stream alone).  A workgroup's partial is stored as fp32 (sum / mean) or, for max, as
+// two 4-byte cells in separate planes: the ordered value and the winner's row.
 
 template <class TR, int VEC, int OP>
 __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
@@ -145,10 +145,15 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
     // this workgroup's partial: [U, C], dense
     const int total = U * C;
     if constexpr (kMax) {
-        unsigned long long *part = reinterpret_cast<unsigned long long *>(partials) + (size_t)blockIdx.x * total;
+        // two planes of 4-byte cells: the ordered values of all workgroups first (all that the
+        // second kernel reads to find the winning partial), the winners' rows behind them
+        unsigned *pval = reinterpret_cast<unsigned *>(partials) + (size_t)blockIdx.x * total;
+        unsigned *prow = reinterpret_cast<unsigned *>(partials) + ((size_t)gridDim.x + blockIdx.x) * total;
         for (int i = threadIdx.x; i < total; i += kTableThreads) {
             const int uu = i / C;
-            part[i] = tkey[uu * stride + (i - uu * C)];
+            const unsigned long long key = tkey[uu * stride + (i - uu * C)];
+            pval[i] = (unsigned)(key >> 32);
+            prow[i] = 0xffffffffu - (unsigned)(key & 0xffffffffull);
         }
     } else {
         float *part = reinterpret_cast<float *>(partials) + (size_t)blockIdx.x * total;
@@ -168,10 +173,11 @@ __global__ __launch_bounds__(kReduceThreads) void table_reduce_kernel(
     const int *__restrict__ preSum, typename TR::raw *__restrict__ out, int *__restrict__ arg,
     int num_parts, int N, int C, int U) {
     constexpr bool kMax = OP == TXS_MAX;
-    using Cell = typename std::conditional<kMax, unsigned long long, float>::type;  // as the forward stored it
+    using Cell = typename std::conditional<kMax, unsigned, float>::type;  // as the forward stored it
+    // max: (ordered value) << 32 | ~workgroup: the largest value wins, among equal values the
+    // first workgroup, whose rows all come before those of the workgroups behind it
     using Acc = typename std::conditional<kMax, unsigned long long, double>::type;
-    // a wave reads whole 128-byte lines of a partial: 16 packed cells or 32 floats
-    constexpr int kSplit = kMax ? kReduceSplit : kReduceSplit / 2;
+    constexpr int kSplit = kReduceSplit;  // a wave reads whole 128-byte lines of a partial: 32 cells
     constexpr int kCellsPerWg = kReduceThreads / kSplit;
     __shared__ Acc part_s[kSplit][kCellsPerWg];
     const int cl = (int)threadIdx.x % kCellsPerWg, wl = (int)threadIdx.x / kCellsPerWg;
@@ -190,7 +196,12 @@ __global__ __launch_bounds__(kReduceThreads) void table_reduce_kernel(
             }
 #pragma unroll
             for (int k = 0; k < kReduceLoads; ++k) {
-                if constexpr (kMax) acc = (Acc)x[k] > acc ? (Acc)x[k] : acc; else acc += (Acc)x[k];
+                if constexpr (kMax) {
+                    const Acc key = ((Acc)x[k] << 32) | (Acc)(0xffffffffu - (unsigned)(w0 + k * kSplit));
+                    acc = key > acc ? key : acc;
+                } else {
+                    acc += (Acc)x[k];
+                }
             }
         }
     }
@@ -217,8 +228,12 @@ __global__ __launch_bounds__(kReduceThreads) void table_reduce_kernel(
     }
     const int u = (int)(cell / C), c = (int)(cell - (long)u * C);
     if constexpr (kMax) {
-        const unsigned row = 0xffffffffu - (unsigned)(acc & 0xffffffffull);
-        if (acc == 0ull || row >= (unsigned)N) {  // no rows, or only NaN: the reference's init pair
+        const unsigned val = (unsigned)(acc >> 32);  // 0: no partial holds a value for this cell
+        const unsigned w = 0xffffffffu - (unsigned)(acc & 0xffffffffull);
+        const unsigned row = (val != 0u && w < (unsigned)num_parts)
+                                 ? reinterpret_cast<const unsigned *>(partials)[((size_t)num_parts + w) * total + cell]
+                                 : 0xffffffffu;
+        if (row >= (unsigned)N) {  // no rows, or only NaN: the reference's init pair
             out[cell] = TR::lowest();
             arg[cell] = -1;
         } else {
@@ -377,7 +392,7 @@ hipError_t launch_table_fwd(const txs_detail::TablePlan &tp, hipStream_t st, con
     kernel<<<dim3(tp.workgroups), dim3(kTableThreads), tp.lds_bytes, st>>>(
         (const raw *)feats, inv, partials, N, C, U, tp.lpr_log2, tp.stride, tp.rows_per_wg);
     const long total = (long)U * C;
-    constexpr int kCellsPerWg = kReduceThreads / (OP == TXS_MAX ? kReduceSplit : kReduceSplit / 2);
+    constexpr int kCellsPerWg = kReduceThreads / kReduceSplit;
     table_reduce_kernel<TR, OP><<<dim3((unsigned)((total + kCellsPerWg - 1) / kCellsPerWg)), dim3(kReduceThreads), 0, st>>>(
         (const raw *)feats, partials, preSum, (raw *)out, arg, tp.workgroups, N, C, U);
     return hipGetLastError();
