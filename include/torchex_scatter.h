@@ -98,8 +98,8 @@ const char *txs_status_string(int status);
 
 /* Name of the kernel instantiation that txs_scatter_forward (backward == 0) or
  * txs_scatter_backward (backward != 0) launches for these extents, as a profiler lists
- * it without namespaces ("scatter_fwd_kernel<F32,4,MAX,16>": dtype, elements per lane,
- * operator, chunk length).  pointer_alignment is
+ * it without namespaces ("scatter_fwd_kernel<F32,4,MAX>": dtype, elements per lane,
+ * operator; "scatter_bwd_kernel<F32,4,MAX,8>": the same and the chunk length).  pointer_alignment is
  * the alignment in bytes of the least aligned tensor (16 for ordinary allocations);
  * table_allowed != 0 means the call would be made with TXS_PATH_AUTO, row-order ids and
  * enough scratch ("table_fwd_kernel<F32,4,MAX>" is then reported where table mode applies).
