@@ -197,6 +197,19 @@ int txs_plan_build_general(const int32_t *unq_inv, int64_t num_total, int64_t nu
 int txs_plan_seg_flag(int32_t *keys_to_seg, int64_t num_total, int64_t num_unq,
                       const int32_t *slot_of, void *stream);
 
+/* Turns the num_heavy heavy voxels at the front of heavy_ids back into ordinary ones: bit 31
+ * comes off their positions in seg, slot_of becomes -1, stats[NUM_HEAVY] = 0 and
+ * stats[NUM_SPECIAL] = stats[NUM_EMPTY]; the caller then passes only the empty voxels as
+ * the special list.  For a plan with a handful of voxels just above the heavy threshold
+ * (a LiDAR sweep in 0.2 m voxels: 8 of 326,859, the fullest with 69 rows): the forward
+ * reduces such runs in registers and LDS like any other, a run may only not reach much
+ * further than the 64 positions a tile stages behind its end (the rest is then read row by
+ * row), and without heavy voxels the forward call needs no second kernel.  (Part of the
+ * index preparation that extends scatter_op.py:13-21; the reference has no heavy voxels.) */
+int txs_plan_demote_heavy(const int32_t *preSum, int32_t *seg, int32_t *slot_of,
+                          const int32_t *heavy_ids, int64_t num_heavy, int64_t num_total,
+                          int64_t num_unq, int32_t *stats, void *stream);
+
 /* seg by binary search of each position in preSum, for callers that hold only
  * CSR offsets of already grouped rows (the reference's scatter_ext.sum /
  * scatter_ext.max argument lists, scatter.cpp:20-53). */

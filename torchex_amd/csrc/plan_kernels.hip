@@ -909,6 +909,22 @@ __global__ void stats_clear_kernel(int *__restrict__ stats) {
     if (threadIdx.x < TXS_STATS_LEN) stats[threadIdx.x] = 0;
 }
 
+// Heavy voxel number blockIdx.x of the list becomes an ordinary one again: the special bit
+// comes off its positions and it gives up its slot.
+__global__ void demote_heavy_kernel(const int *__restrict__ preSum, int *__restrict__ seg,
+                                    int *__restrict__ slot_of, const int *__restrict__ heavy_ids,
+                                    int N, int U, int *__restrict__ stats) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        stats[TXS_STAT_NUM_HEAVY] = 0;
+        stats[TXS_STAT_NUM_SPECIAL] = stats[TXS_STAT_NUM_EMPTY];
+    }
+    const int u = heavy_ids[blockIdx.x];
+    if ((unsigned)u >= (unsigned)U) return;
+    const int lo = max(preSum[u], 0), hi = min(preSum[u + 1], N);
+    for (int p = lo + (int)threadIdx.x; p < hi; p += (int)blockDim.x) seg[p] &= kIdMask;
+    if (threadIdx.x == 0) slot_of[u] = -1;
+}
+
 int radix_bits(int64_t U) {
     int bits = 1;
     while ((1LL << bits) < U) ++bits;
@@ -1017,6 +1033,17 @@ int txs_plan_seg_flag(int32_t *keys_to_seg, int64_t num_total, int64_t num_unq,
     if (!keys_to_seg || !slot_of) return TXS_ERR_INVALID_ARG;
     seg_flag_kernel<<<dim3(blocks_for(num_total)), dim3(kThreads), 0, (hipStream_t)stream>>>(
         keys_to_seg, num_total, (int)num_unq, slot_of, keys_to_seg);
+    return status_of(hipGetLastError());
+}
+
+int txs_plan_demote_heavy(const int32_t *preSum, int32_t *seg, int32_t *slot_of, const int32_t *heavy_ids,
+                          int64_t num_heavy, int64_t num_total, int64_t num_unq, int32_t *stats, void *stream) {
+    if (!fits_i32(num_total) || !fits_i32(num_unq) || num_heavy < 0 || num_heavy > num_unq)
+        return TXS_ERR_INVALID_ARG;
+    if (num_heavy == 0) return TXS_OK;
+    if (!preSum || !seg || !slot_of || !heavy_ids || !stats) return TXS_ERR_INVALID_ARG;
+    demote_heavy_kernel<<<dim3((unsigned)num_heavy), dim3(128), 0, (hipStream_t)stream>>>(
+        preSum, seg, slot_of, heavy_ids, (int)num_total, (int)num_unq, stats);
     return status_of(hipGetLastError());
 }
 

@@ -88,6 +88,25 @@ Tensor special_list(const Tensor &heavy_all, int64_t capacity, const std::vector
     return at::cat({heavy, heavy_all.narrow(0, capacity - n_empty, n_empty)});
 }
 
+// A handful of voxels just above the default heavy threshold are not worth the heavy path:
+// the forward kernel reduces a run a little longer than the 64 positions a tile stages behind
+// its end like any other (the last few rows one by one), and a plan without heavy voxels saves
+// every forward call its second kernel.  A threshold chosen by the caller is left alone.
+constexpr int64_t kDemoteMostVoxels = 64;  // heavy voxels at most ...
+constexpr int64_t kDemoteLongest = 96;     // ... none of them longer than this
+void demote_few_heavy(std::vector<int64_t> &hs, int64_t heavy_threshold, const Tensor &preSum, Tensor &seg,
+                      Tensor &slot_of, const Tensor &heavy_all, Tensor &stats, int64_t N, int64_t U, void *st) {
+    const int64_t n_heavy = hs[TXS_STAT_NUM_HEAVY];
+    if (heavy_threshold != txs_default_heavy_threshold() || n_heavy == 0 || n_heavy > kDemoteMostVoxels ||
+        hs[TXS_STAT_MAX_CNT] > kDemoteLongest || hs[TXS_STAT_OUT_OF_RANGE])
+        return;
+    check_status(txs_plan_demote_heavy(i32p(preSum), i32w(seg), i32w(slot_of), i32p(heavy_all), n_heavy, N, U,
+                                       i32w(stats), st),
+                 "plan_demote_heavy");
+    hs[TXS_STAT_NUM_HEAVY] = 0;
+    hs[TXS_STAT_NUM_SPECIAL] = hs[TXS_STAT_NUM_EMPTY];
+}
+
 // ScatterData index preparation for an unq_inv in any order
 // (extends torchex/operator_py/scatter_op.py:13-21).  Everything is queued on
 // the current stream; the only host synchronisation is the read of `stats`.
@@ -148,6 +167,7 @@ std::tuple<Tensor, OptTensor, Tensor, Tensor, Tensor, std::vector<int64_t>> buil
                 "unq_inv holds ids outside [0, num_unq=", U, ")");
     TORCH_CHECK(!(assume_sorted && hs[TXS_STAT_UNSORTED]),
                 "unq_inv was declared sorted (assume_sorted=True) but is not non-decreasing");
+    demote_few_heavy(hs, heavy_threshold, preSum, seg, slot_of, heavy_all, stats, N, U, st);
     OptTensor perm_out;
     if (hs[TXS_STAT_UNSORTED]) perm_out = perm;
     Tensor heavy_ids = special_list(heavy_all, U, hs);
@@ -174,6 +194,7 @@ std::tuple<Tensor, Tensor, Tensor, std::vector<int64_t>> plan_from_presum(
         check_status(txs_plan_seg_from_presum(i32p(preSum), N, U, i32p(slot_of), i32w(seg), st),
                      "plan_seg_from_presum");
     std::vector<int64_t> hs = read_stats(stats);
+    if (U > 0) demote_few_heavy(hs, heavy_threshold, preSum, seg, slot_of, heavy_all, stats, N, U, st);
     Tensor heavy_ids = special_list(heavy_all, U, hs);
     return {seg, slot_of, heavy_ids, hs};
 }
@@ -277,6 +298,7 @@ unique_plan(const Tensor &keys_in, int64_t key_bound, int64_t heavy_threshold, c
     TORCH_CHECK(hs[TXS_STAT_OUT_OF_RANGE] == 0, "keys (or points) outside the grid: keys must be in [0, ",
                 key_bound, ")");
     const int64_t U = hs[TXS_STAT_NUM_UNQ];
+    demote_few_heavy(hs, heavy_threshold, preSum, seg, slot_of, heavy_all, stats, N, U, st);
     OptTensor perm_out;
     if (hs[TXS_STAT_UNSORTED]) perm_out = perm;
     return {unq.narrow(0, 0, U), inv, cnts.narrow(0, 0, U), preSum.narrow(0, 0, U + 1), perm_out, seg,
