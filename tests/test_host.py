@@ -40,7 +40,7 @@ def test_header_is_plain_c_and_links(tmp_path):
         pytest.skip("no C compiler on this machine")
     src = tmp_path / "abi.c"
     src.write_text('#include "torchex_scatter.h"\n'
-                   'int main(void) { return txs_abi_version() == 8 && txs_chunk_rows() > 0 ? 0 : 1; }\n')
+                   'int main(void) { return txs_abi_version() == 9 && txs_chunk_rows() > 0 ? 0 : 1; }\n')
     inc = os.path.join(ROOT, "include")
     pkg = os.path.join(ROOT, "torchex_amd")
     subprocess.check_call([cc, "-std=c11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I" + inc,
@@ -53,7 +53,7 @@ def test_header_is_plain_c_and_links(tmp_path):
 
 def test_host_only_entry_points():
     lib = _lib()
-    assert lib.txs_abi_version() == 8
+    assert lib.txs_abi_version() == 9
     lib.txs_status_string.restype = ctypes.c_char_p
     assert lib.txs_status_string(0) == b"ok"
     assert b"invalid" in lib.txs_status_string(1)

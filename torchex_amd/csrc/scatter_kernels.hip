@@ -980,7 +980,7 @@ int scatter_forward_impl(int op, int dtype, const void *feats, const int32_t *un
 
 extern "C" {
 
-int txs_abi_version(void) { return 8; }
+int txs_abi_version(void) { return 9; }
 
 const char *txs_status_string(int status) {
     switch (status) {
