@@ -150,8 +150,9 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     int b_lo = bnd_s[0], b_hi = bnd_s[1];
     const int l_staged_end = n_seg_s;  // one past the last staged l
     if (b_lo < 0) {
-        // an ordinary run of more than kMargin rows covers the tile's first positions (only a
-        // plan with a heavy threshold above kMargin has one): look for its end one by one
+        // an ordinary run of more than kMargin rows covers the tile's first positions (a plan
+        // with a heavy threshold above kMargin has such runs, and so has one whose few voxels
+        // just above the threshold were made ordinary again): look for its end one by one
         b_lo = kMargin + 1;
         while (b_lo < l_staged_end && seg_s[b_lo] == seg_s[b_lo - 1] && seg_s[b_lo] >= 0) ++b_lo;
     }
