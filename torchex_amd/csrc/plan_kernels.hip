@@ -873,8 +873,8 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
         }
         __syncthreads();
         // destination = slice-start position of the voxel + rows of the voxel that the waves
-        // in front of this one hold in this round + rank inside the wave; the per-voxel
-        // bookkeeping is done per ROW (a few LDS operations each), never per voxel: a round
+        // in front of this one hold in this pass + rank inside the wave; the per-voxel
+        // bookkeeping is done per ROW (a few LDS operations each), never per voxel: a pass
         // has fewer rows than a bucket can have voxel-times-wave counters
         long dst[kBktItems];
 #pragma unroll
@@ -891,7 +891,7 @@ __global__ __launch_bounds__(kThreads) void bucket_plan_kernel(
         for (int it = 0; it < kBktItems; ++it) {
             if (key[it] < 0) continue;
             const int dg = key[it] - u_lo;
-            atomicAdd(&off[dg], 1);       // the next round starts behind this round's rows
+            atomicAdd(&off[dg], 1);       // the next pass starts behind this pass's rows
             wc[w * low_bins + dg] = 0;    // (every row of the group stores the same zero)
             if (rank_mode) {
                 if ((unsigned)row[it] < (unsigned)n) ranks[row[it]] = (long long)(dst[it] - s);

@@ -139,7 +139,7 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
             }
         }
         // position p + 1 (l = e + 1) can open a range: a run starts there, or it is heavy
-        const int eb = e0 + ((int)threadIdx.x & ~63);  // first entry of this wave in this round
+        const int eb = e0 + ((int)threadIdx.x & ~63);  // first entry of this wave in this pass of the loop
         if (eb == 0 || eb == T) {
             const unsigned long long m = __ballot(e < n_seg_s && (sn != sv || (sn < 0)));
             if (((int)threadIdx.x & 63) == 0)

@@ -142,24 +142,52 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
         }
     }
     __syncthreads();
-    // this workgroup's partial: [U, C], dense
+    // this workgroup's partial: [U, C], dense; four cells per lane and store where the row
+    // length and the partial's address allow 16-byte stores
     const int total = U * C;
+    const bool wide = (C & 3) == 0 && (reinterpret_cast<size_t>(partials) & 15) == 0;
     if constexpr (kMax) {
         // two planes of 4-byte cells: the ordered values of all workgroups first (all that the
         // second kernel reads to find the winning partial), the winners' rows behind them
         unsigned *pval = reinterpret_cast<unsigned *>(partials) + (size_t)blockIdx.x * total;
         unsigned *prow = reinterpret_cast<unsigned *>(partials) + ((size_t)gridDim.x + blockIdx.x) * total;
-        for (int i = threadIdx.x; i < total; i += kTableThreads) {
-            const int uu = i / C;
-            const unsigned long long key = tkey[uu * stride + (i - uu * C)];
-            pval[i] = (unsigned)(key >> 32);
-            prow[i] = 0xffffffffu - (unsigned)(key & 0xffffffffull);
+        if (wide) {
+            for (int i = (int)threadIdx.x * 4; i < total; i += kTableThreads * 4) {
+                const int uu = i / C;
+                const unsigned long long *t = tkey + uu * stride + (i - uu * C);
+                Pack<unsigned, 4> v, r;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v.v[e] = (unsigned)(t[e] >> 32);
+                    r.v[e] = 0xffffffffu - (unsigned)(t[e] & 0xffffffffull);
+                }
+                st<unsigned, 4>(pval + i, v);
+                st<unsigned, 4>(prow + i, r);
+            }
+        } else {
+            for (int i = threadIdx.x; i < total; i += kTableThreads) {
+                const int uu = i / C;
+                const unsigned long long key = tkey[uu * stride + (i - uu * C)];
+                pval[i] = (unsigned)(key >> 32);
+                prow[i] = 0xffffffffu - (unsigned)(key & 0xffffffffull);
+            }
         }
     } else {
         float *part = reinterpret_cast<float *>(partials) + (size_t)blockIdx.x * total;
-        for (int i = threadIdx.x; i < total; i += kTableThreads) {
-            const int uu = i / C;
-            part[i] = (float)tsum[uu * stride + (i - uu * C)];
+        if (wide) {
+            for (int i = (int)threadIdx.x * 4; i < total; i += kTableThreads * 4) {
+                const int uu = i / C;
+                const double *t = tsum + uu * stride + (i - uu * C);
+                Pack<float, 4> v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v.v[e] = (float)t[e];
+                st<float, 4>(part + i, v);
+            }
+        } else {
+            for (int i = threadIdx.x; i < total; i += kTableThreads) {
+                const int uu = i / C;
+                part[i] = (float)tsum[uu * stride + (i - uu * C)];
+            }
         }
     }
 }
