@@ -292,26 +292,65 @@ __global__ __launch_bounds__(kTableThreads) void table_bwd_kernel(
                                       (((size_t)U * stride * sizeof(raw) + 31) & ~(size_t)31));
     const int total = U * C;
     constexpr int kStage = 4;  // independent loads per lane while the tables are staged
-    for (int i0 = threadIdx.x; i0 < total; i0 += kTableThreads * kStage) {
-        raw x[kStage];
-        int a[kStage], cnt[kStage], uu[kStage];
+    // one cell of the staged tables: upstream value (mean: divided by the voxel's count, one
+    // division per output cell as (g / unq_cnts) in the reference) and, for max, the winner
+    auto staged = [&](raw x, int cnt) -> raw {
+        return OP == TXS_MEAN ? TR::from_f(TR::to_f(x) / (float)cnt) : x;
+    };
+    if constexpr (VEC * sizeof(raw) >= 4) {
+        // VEC cells per lane and load (C is a multiple of VEC and every tensor is aligned to
+        // the lane's bytes; arg rows, 4 bytes per cell, go in pieces of that many bytes)
+        constexpr int kArgPiece = VEC * (int)sizeof(raw) / 4;  // ints per piece
+        constexpr int kArgPieces = VEC / kArgPiece;
+        for (int i0 = (int)threadIdx.x * VEC; i0 < total; i0 += kTableThreads * VEC * kStage) {
+            Pack<raw, VEC> x[kStage];
+            Pack<int, kArgPiece> a[kStage][kArgPieces];
+            int cnt[kStage], uu[kStage];
 #pragma unroll
-        for (int k = 0; k < kStage; ++k) {
-            const int i = min(i0 + k * kTableThreads, total - 1);
-            uu[k] = i / C;
-            x[k] = g[i];
-            if (OP == TXS_MEAN) cnt[k] = preSum[uu[k] + 1] - preSum[uu[k]];
-            if (OP == TXS_MAX) a[k] = arg[i];
+            for (int k = 0; k < kStage; ++k) {
+                const int i = min(i0 + k * kTableThreads * VEC, total - VEC);
+                uu[k] = i / C;
+                x[k] = ld<raw, VEC>(g + i);
+                if (OP == TXS_MEAN) cnt[k] = preSum[uu[k] + 1] - preSum[uu[k]];
+                if (OP == TXS_MAX) {
+#pragma unroll
+                    for (int q = 0; q < kArgPieces; ++q) a[k][q] = ld<int, kArgPiece>(arg + i + q * kArgPiece);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < kStage; ++k) {
+                const int i = i0 + k * kTableThreads * VEC;
+                if (i >= total) break;
+                const int cell = uu[k] * stride + (i - uu[k] * C);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) x[k].v[e] = staged(x[k].v[e], OP == TXS_MEAN ? cnt[k] : 1);
+                st<raw, VEC>(gt + cell, x[k]);
+                if (OP == TXS_MAX) {
+#pragma unroll
+                    for (int q = 0; q < kArgPieces; ++q) st<int, kArgPiece>(at + cell + q * kArgPiece, a[k][q]);
+                }
+            }
         }
+    } else {
+        for (int i0 = threadIdx.x; i0 < total; i0 += kTableThreads * kStage) {
+            raw x[kStage];
+            int a[kStage], cnt[kStage], uu[kStage];
 #pragma unroll
-        for (int k = 0; k < kStage; ++k) {
-            const int i = i0 + k * kTableThreads;
-            if (i >= total) break;
-            const int c = i - uu[k] * C;
-            if (OP == TXS_MEAN)  // one division per output cell, as (g / unq_cnts) in the reference
-                x[k] = TR::from_f(TR::to_f(x[k]) / (float)cnt[k]);
-            gt[uu[k] * stride + c] = x[k];
-            if (OP == TXS_MAX) at[uu[k] * stride + c] = a[k];
+            for (int k = 0; k < kStage; ++k) {
+                const int i = min(i0 + k * kTableThreads, total - 1);
+                uu[k] = i / C;
+                x[k] = g[i];
+                if (OP == TXS_MEAN) cnt[k] = preSum[uu[k] + 1] - preSum[uu[k]];
+                if (OP == TXS_MAX) a[k] = arg[i];
+            }
+#pragma unroll
+            for (int k = 0; k < kStage; ++k) {
+                const int i = i0 + k * kTableThreads;
+                if (i >= total) break;
+                const int c = i - uu[k] * C;
+                gt[uu[k] * stride + c] = staged(x[k], OP == TXS_MEAN ? cnt[k] : 1);
+                if (OP == TXS_MAX) at[uu[k] * stride + c] = a[k];
+            }
         }
     }
     __syncthreads();
