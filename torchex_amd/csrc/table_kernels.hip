@@ -44,7 +44,10 @@ constexpr int kTableLdsBudget = 144 * 1024;  // bytes of LDS a table may take (1
 constexpr int kTableUnroll = TXS_TABLE_UNROLL;  // rows per lane in flight (twice as many for lanes of 4 bytes or less in the forward)
 constexpr int kReduceThreads = 1024;
 constexpr int kReduceSplit = 32;             // lanes that share the partials of one output cell
-constexpr int kReduceLoads = 4;              // partials each of them has in flight
+#ifndef TXS_REDUCE_LOADS
+#define TXS_REDUCE_LOADS 4
+#endif
+constexpr int kReduceLoads = TXS_REDUCE_LOADS;  // partials each of them has in flight
 
 // ------------------------------------------------------------------ forward --
 //
@@ -67,8 +70,6 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
     unsigned long long *tkey = table_lds;
     double *tsum = reinterpret_cast<double *>(table_lds);
     const int cells = U * stride;
-    for (int i = threadIdx.x; i < cells; i += kTableThreads) tkey[i] = 0ull;  // +0.0 as a double
-    __syncthreads();
 
     const int lane_in = (int)threadIdx.x & ((1 << lpr_log2) - 1);
     const int g = (int)threadIdx.x >> lpr_log2;
@@ -76,7 +77,7 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
     const int col = lane_in * VEC;
     const long r0 = (long)blockIdx.x * rows_per_wg;
     const int r_end = (int)min((long)N, r0 + rows_per_wg);
-    if (col < C) {
+    {
         // Two batches of kRows rows per lane: the next one is on its way from memory
         // while the current one goes into the table.
         struct Batch {
@@ -120,9 +121,12 @@ __global__ __launch_bounds__(kTableThreads) void table_fwd_kernel(
             }
         };
         int rb = (int)r0 + g;
-        if (rb < r_end) {
-            Batch b0, b1;
-            issue(b0, rb);
+        const bool act = col < C && rb < r_end;
+        Batch b0, b1;
+        if (act) issue(b0, rb);  // the first rows are on their way while the table is cleared
+        for (int i = threadIdx.x; i < cells; i += kTableThreads) tkey[i] = 0ull;  // +0.0 as a double
+        __syncthreads();
+        if (act) {
             for (;;) {
                 if (rb + step >= r_end) {
                     consume(b0, rb);
@@ -290,6 +294,24 @@ __global__ __launch_bounds__(kTableThreads) void table_bwd_kernel(
     // arg rows follow the upstream rows, 32-byte aligned
     int *at = reinterpret_cast<int *>(reinterpret_cast<char *>(table_lds) +
                                       (((size_t)U * stride * sizeof(raw) + 31) & ~(size_t)31));
+    const int lane_in = (int)threadIdx.x & ((1 << lpr_log2) - 1);
+    const int grp = (int)threadIdx.x >> lpr_log2;
+    const int G = kTableThreads >> lpr_log2;
+    const int col = lane_in * VEC;
+    const long r0 = (long)blockIdx.x * rows_per_wg;
+    const int r_end = (int)min((long)N, r0 + rows_per_wg);
+    // the voxel ids of the next batch of rows are fetched while the current batch is written
+    // (and those of the first batch while the tables are staged)
+    const int step = G * kTableUnroll;
+    auto issue = [&](int (&u)[kTableUnroll], int rb) {
+#pragma unroll
+        for (int k = 0; k < kTableUnroll; ++k) u[k] = inv[min(rb + k * G, r_end - 1)] & kIdMask;
+    };
+    int rb = (int)r0 + grp;
+    const bool act = col < C && rb < r_end;
+    int u0[kTableUnroll], u1[kTableUnroll];
+    if (act) issue(u0, rb);
+
     const int total = U * C;
     constexpr int kStage = 4;  // independent loads per lane while the tables are staged
     // one cell of the staged tables: upstream value (mean: divided by the voxel's count, one
@@ -355,19 +377,7 @@ __global__ __launch_bounds__(kTableThreads) void table_bwd_kernel(
     }
     __syncthreads();
 
-    const int lane_in = (int)threadIdx.x & ((1 << lpr_log2) - 1);
-    const int grp = (int)threadIdx.x >> lpr_log2;
-    const int G = kTableThreads >> lpr_log2;
-    const int col = lane_in * VEC;
-    if (col >= C) return;
-    const long r0 = (long)blockIdx.x * rows_per_wg;
-    const int r_end = (int)min((long)N, r0 + rows_per_wg);
-    // the voxel ids of the next batch of rows are fetched while the current batch is written
-    const int step = G * kTableUnroll;
-    auto issue = [&](int (&u)[kTableUnroll], int rb) {
-#pragma unroll
-        for (int k = 0; k < kTableUnroll; ++k) u[k] = inv[min(rb + k * G, r_end - 1)] & kIdMask;
-    };
+    if (!act) return;
     auto emit = [&](const int (&u)[kTableUnroll], int rb) {
 #pragma unroll
         for (int k = 0; k < kTableUnroll; ++k) {
@@ -388,10 +398,6 @@ __global__ __launch_bounds__(kTableThreads) void table_bwd_kernel(
             if (TXS_TABLE_NT_STORES) st_stream<raw, VEC>(gin + (size_t)r * C + col, o); else st<raw, VEC>(gin + (size_t)r * C + col, o);
         }
     };
-    int rb = (int)r0 + grp;
-    if (rb >= r_end) return;
-    int u0[kTableUnroll], u1[kTableUnroll];
-    issue(u0, rb);
     for (;;) {
         if (rb + step >= r_end) {
             emit(u0, rb);
