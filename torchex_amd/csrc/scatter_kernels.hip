@@ -518,23 +518,40 @@ __global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
     emit(std::false_type{}, head_seg, hacc, hidx, cnt, (long)t0 - 1 + first_l, (long)t0 + head_l);
 }
 
-// Turn the scratch table of the special voxels into output rows and clear it.
+// Turn the scratch table of the special voxels into output rows and clear it.  The first
+// n_heavy entries of heavy_ids are the heavy voxels (entry s owns table row s), the rest are
+// empty voxels, which own no row: a cell's table word does not depend on the voxel's id, so
+// it is requested together with the id, and only the mean goes on to the voxel's count.
 template <class TR, int OP>
 __global__ void scatter_finalize_kernel(const typename TR::raw *__restrict__ feats,
                                         const int *__restrict__ preSum,
                                         const int *__restrict__ heavy_ids,
                                         unsigned long long *__restrict__ scratch,
                                         typename TR::raw *__restrict__ out,
-                                        int *__restrict__ arg, int n_special, int N, int C, int U,
-                                        const int *__restrict__ perm, int ref_log2) {
+                                        int *__restrict__ arg, int n_special, int n_heavy, int N, int C,
+                                        int U, const int *__restrict__ perm, int ref_log2) {
+    constexpr bool kMaxOp = OP == TXS_MAX || OP == TXS_MAX_REFTIE;
     const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= (long)n_special * C) return;
     const int s = (int)(t / C), c = (int)(t - (long)s * C);
+    const bool heavy = s < n_heavy;
+    unsigned long long key = 0ull;
+    float s32 = 0.0f;
+    if (heavy) {
+        if (kMaxOp) {
+            key = scratch[t];
+            scratch[t] = 0ull;
+        } else {
+            float *fs = reinterpret_cast<float *>(scratch);
+            s32 = fs[t];
+            fs[t] = 0.0f;
+        }
+    }
     const int u = heavy_ids[s];
     if ((unsigned)u >= (unsigned)U) return;
     const size_t o = (size_t)u * C + c;
-    if (preSum[u + 1] == preSum[u]) {  // empty voxel: listed after the heavy ones, owns no scratch row
-        if (OP == TXS_MAX || OP == TXS_MAX_REFTIE) {
+    if (!heavy) {  // empty voxel
+        if (kMaxOp) {
             out[o] = TR::lowest();
             arg[o] = -1;
         } else {
@@ -542,9 +559,7 @@ __global__ void scatter_finalize_kernel(const typename TR::raw *__restrict__ fea
         }
         return;
     }
-    if (OP == TXS_MAX || OP == TXS_MAX_REFTIE) {
-        const unsigned long long key = scratch[t];
-        scratch[t] = 0ull;
+    if (kMaxOp) {
         unsigned row = 0xffffffffu - (unsigned)(key & 0xffffffffull);
         if (OP == TXS_MAX_REFTIE && key != 0ull) {  // the low word holds a tie key, not a row
             const long pos = (long)preSum[u] + ref_rel((int)row, ref_log2);
@@ -561,9 +576,6 @@ __global__ void scatter_finalize_kernel(const typename TR::raw *__restrict__ fea
             arg[o] = (int)row;
         }
     } else {
-        float *fs = reinterpret_cast<float *>(scratch);
-        float s32 = fs[t];
-        fs[t] = 0.0f;
         if (OP == TXS_MEAN) s32 = s32 / (float)(preSum[u + 1] - preSum[u]);
         out[o] = TR::from_f(s32);
     }
@@ -801,7 +813,7 @@ hipError_t launch_fwd(int op, const Geometry &geo, hipStream_t st, const void *f
 template <class TR>
 hipError_t launch_finalize(int op, hipStream_t st, const void *feats, const int *preSum,
                            const int *heavy_ids, void *scratch, void *out, int *arg,
-                           long n_special, int N, int C, int U, const int *perm, int ref_log2) {
+                           long n_special, long n_heavy, int N, int C, int U, const int *perm, int ref_log2) {
     using raw = typename TR::raw;
     const long total = n_special * C;
     if (total <= 0) return hipSuccess;
@@ -812,19 +824,19 @@ hipError_t launch_finalize(int op, hipStream_t st, const void *feats, const int 
     switch (op) {
         case TXS_SUM:
             scatter_finalize_kernel<TR, TXS_SUM><<<grid, blk, 0, st>>>(f, preSum, heavy_ids, s, o, arg,
-                                                                      (int)n_special, N, C, U, perm, ref_log2);
+                                                                      (int)n_special, (int)n_heavy, N, C, U, perm, ref_log2);
             break;
         case TXS_MEAN:
             scatter_finalize_kernel<TR, TXS_MEAN><<<grid, blk, 0, st>>>(f, preSum, heavy_ids, s, o, arg,
-                                                                       (int)n_special, N, C, U, perm, ref_log2);
+                                                                       (int)n_special, (int)n_heavy, N, C, U, perm, ref_log2);
             break;
         case TXS_MAX_REFTIE:
             scatter_finalize_kernel<TR, TXS_MAX_REFTIE><<<grid, blk, 0, st>>>(
-                f, preSum, heavy_ids, s, o, arg, (int)n_special, N, C, U, perm, ref_log2);
+                f, preSum, heavy_ids, s, o, arg, (int)n_special, (int)n_heavy, N, C, U, perm, ref_log2);
             break;
         default:
             scatter_finalize_kernel<TR, TXS_MAX><<<grid, blk, 0, st>>>(f, preSum, heavy_ids, s, o, arg,
-                                                                      (int)n_special, N, C, U, perm, ref_log2);
+                                                                      (int)n_special, (int)n_heavy, N, C, U, perm, ref_log2);
             break;
     }
     return hipGetLastError();
@@ -966,11 +978,11 @@ int scatter_forward_impl(int op, int dtype, const void *feats, const int32_t *un
     }
     if (num_special > 0) {
         if (dtype == TXS_F32)
-            e = launch_finalize<F32>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U, perm, ref_log2);
+            e = launch_finalize<F32>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, num_heavy, N, C, U, perm, ref_log2);
         else if (dtype == TXS_F16)
-            e = launch_finalize<F16>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U, perm, ref_log2);
+            e = launch_finalize<F16>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, num_heavy, N, C, U, perm, ref_log2);
         else
-            e = launch_finalize<BF16>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, N, C, U, perm, ref_log2);
+            e = launch_finalize<BF16>(op, st, feats, preSum, heavy_ids, scratch, out, arg, num_special, num_heavy, N, C, U, perm, ref_log2);
     }
     return status_of(e);
 }
