@@ -86,8 +86,18 @@ __device__ __forceinline__ int ref_rel(int key, int blog2) {  // inverse of ref_
     return (int)((iter << blog2) | ref_prio((unsigned)key >> kIterBits, blog2 - 5));
 }
 
+// Waves per SIMD the compiler has to make room for: the fp16 max/argmax kernel comes out at 84
+// registers (allocated in eights: 5 waves) and is the one forward kernel that gains from a
+// sixth (80 registers and three spilled dwords; pillar binning: 76-79 -> 73-75 us); asked of
+// the fp32 max it spills in earnest (152 -> 202 us), so it is asked of that kernel only.
+template <class TR, int OP>
+constexpr int fwd_min_waves() {
+    return (std::is_same<TR, F16>::value && OP == TXS_MAX) ? 6 : 1;
+}
+
 template <class TR, int VEC, int OP>
-__global__ __launch_bounds__(kThreads) void scatter_fwd_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(fwd_min_waves<TR, OP>(), 8)))
+void scatter_fwd_kernel(
     const typename TR::raw *__restrict__ feats, const int *__restrict__ perm,
     const int *__restrict__ seg, const int *__restrict__ slot_of,
     typename TR::raw *__restrict__ out, int *__restrict__ arg,
