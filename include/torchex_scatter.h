@@ -108,8 +108,9 @@ int txs_kernel_name(int backward, int op, int dtype, int64_t num_total, int64_t 
                     int64_t num_unq, int64_t pointer_alignment, int table_allowed, char *buf,
                     int64_t buf_len);
 
-/* Default population above which a voxel is reduced through atomics, and the
- * number of sorted positions one lane group walks. */
+/* Default population above which a voxel is reduced through atomics (64), and the
+ * smallest heavy_threshold the plan functions accept (16: a smaller one is refused with
+ * TXS_ERR_INVALID_ARG). */
 int txs_default_heavy_threshold(void);
 int txs_chunk_rows(void);
 

@@ -384,6 +384,40 @@ def test_few_short_heavy_voxels_stay_ordinary(dtype):
     assert data.num_heavy == 65
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_seeded_shapes(seed):
+    """Shapes nobody chose by hand: channel counts that leave lanes idle or need a second
+    column block, run lengths from geometric, uniform and heavy-tailed draws, thresholds on
+    both sides of the run lengths, all three dtypes, grouped and shuffled rows, empty voxels."""
+    g = torch.Generator().manual_seed(9000 + seed)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+
+    C = [1, 2, 3, 5, 7, 8, 12, 16, 24, 31, 32, 48, 64, 96, 100, 128, 160, 200, 256, 257, 300, 384, 512, 6][seed]
+    U = ri(1, 4000)
+    kind = seed % 3
+    if kind == 0:      # short runs, some empty voxels
+        cnts = torch.poisson(torch.full((U,), 1.5), generator=g).long()
+    elif kind == 1:    # up to a few tiles long
+        cnts = torch.randint(0, 3 * ri(8, 200), (U,), generator=g)
+    else:              # heavy tail
+        cnts = (torch.rand((U,), generator=g) ** 6 * ri(100, 3000)).long() + torch.randint(0, 2, (U,), generator=g)
+    if int(cnts.sum()) == 0:
+        cnts[0] = 1
+    budget = 6_000_000 // C                      # rows the oracle gets through in a second or two
+    while int(cnts.sum()) > budget:
+        cnts = cnts // 2
+    inv_sorted = torch.repeat_interleave(torch.arange(U), cnts)
+    N = inv_sorted.numel()
+    feats = torch.randn((N, C), generator=g)
+    feats[torch.rand((N, C), generator=g) < 0.03] = 0.75       # ties
+    thr = [None, 16, 32, 64, 100, 5000][ri(0, 5)]     # (16 is the smallest the library accepts)
+    dtype = [torch.float32, torch.float16, torch.bfloat16][ri(0, 2)]
+    inv = inv_sorted if seed % 4 == 0 else inv_sorted[torch.randperm(N, generator=g)]
+    run_case(f"seeded_{seed}", feats, inv, cnts, dtype=dtype, heavy_threshold=thr, grad_seed=300 + seed)
+
+
 # ------------------------------------------------- the reference's own test --
 
 def test_reference_test_data_closed_forms(reference_counts):
