@@ -1215,7 +1215,7 @@ def test_zipf_contention_takes_the_table_kernels_and_both_paths_agree():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("C", [1, 3, 4, 16, 20, 64])
+@pytest.mark.parametrize("C", [1, 2, 3, 4, 6, 10, 16, 20, 24, 64])
 def test_table_kernels_channel_widths_and_dtypes(C, dtype):
     from torchex_amd._native import scatter_ext
     g = torch.Generator().manual_seed(500 + C)
