@@ -96,6 +96,54 @@ def test_from_keys_equals_torch_unique_and_scatter_data(case):
     assert torch.equal(fg.grad, (1.0 / cnt.float()).to(DEV)[inv.to(DEV)].unsqueeze(1).expand(-1, 16))
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_from_keys_seeded(seed):
+    """Key sets nobody chose by hand: grids smaller and far larger than the input (both routes
+    of from_keys), dense, clustered and heavy-tailed occupancy, int32 and int64 keys."""
+    T = tx()
+    g = torch.Generator().manual_seed(4000 + seed)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+
+    N = [1, 7, 300, 5_000, 40_000, 120_000, 250_000, 33_333, 65_536, 65_537, 99_999, 500_000][seed]
+    bound = [1, 3, 10_000, 2**31 - 32770, 1_000, 7_000_000, 100_000, 2**20, 70_000, 12_345_678, 64, 20_000_000][seed]
+    kind = seed % 3
+    if kind == 0:
+        keys = torch.randint(0, bound, (N,), generator=g)
+    elif kind == 1:      # clustered: a few hundred distinct keys, some of them crowded
+        pool = torch.randint(0, bound, (min(bound, ri(1, 300)),), generator=g)
+        keys = pool[(torch.rand((N,), generator=g) ** 3 * pool.numel()).long()]
+    else:                # mostly distinct, with runs of equal neighbours
+        keys = torch.randint(0, bound, (N,), generator=g)
+        keys[1::2] = keys[0::2][: keys[1::2].numel()]
+    if seed % 2:
+        keys = keys.int()
+    if seed == 3:        # one past the largest key bound the library takes
+        with pytest.raises(RuntimeError):
+            T.ScatterData.from_keys(keys.to(DEV), bound + 1)
+    say(f"[case] from_keys seeded {seed} N={N} bound={bound} dtype={keys.dtype}")
+    unq, inv, cnt = torch.unique(keys.long(), return_inverse=True, return_counts=True)
+    data = T.ScatterData.from_keys(keys.to(DEV), bound)
+    assert torch.equal(data.unq_keys.cpu().long(), unq)
+    assert torch.equal(data.unq_inv.cpu().long(), inv)
+    assert torch.equal(data.unq_cnts.cpu().reshape(-1), cnt)
+    assert data.num_unq == unq.shape[0] and data.max_cnt == int(cnt.max())
+    inv32 = inv.numpy().astype(np.int32)
+    pre = orc.presum(cnt.numpy())
+    assert np.array_equal(data.preSum.cpu().numpy(), pre)
+    perm = data.perm.cpu().numpy() if data.perm is not None else np.arange(N, dtype=np.int32)
+    assert np.array_equal(perm, orc.stable_perm(inv32, pre))
+    assert np.array_equal(data.seg.cpu().numpy() & 0x7fffffff, inv32[perm])
+    # the plan drives the operators as the plan of ScatterData(torch.unique(...)) does
+    feats = torch.randn((N, 8), generator=g).to(DEV)
+    ref = T.ScatterData(inv.to(DEV), cnt.to(DEV))
+    assert (data.num_special, data.num_heavy) == (ref.num_special, ref.num_heavy)
+    a, b = T.scatter_max(feats, data), T.scatter_max(feats, ref)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    assert np.array_equal(T.ingroup_inds(keys.to(DEV)).cpu().numpy(), orc.ingroup_inds(keys.long().numpy()))
+
+
 def test_from_keys_occupancy_map_and_sort_agree():
     """from_keys numbers the keys with an occupancy map of the grid when the grid is not much
     larger than the input and sorts them otherwise.  The same keys under a small and under a huge
