@@ -58,6 +58,11 @@ class ScatterData:
     voxel at each sorted position, bit 31 marking voxels reduced through
     atomics), ``slot_of`` / ``heavy_ids`` (table of those voxels).
 
+    ``heavy_threshold`` (default 64, at least 16): voxels with more rows are reduced
+    through atomics.  With the default, a plan whose only heavy voxels are a handful just
+    above it (at most 64 of them, none above 96 rows) keeps them ordinary, so that a
+    forward call is a single kernel; ``num_heavy`` is then 0.
+
     ``max_tie_rule``: ``"reference"`` reports, among equal maxima, the row the reference
     kernel reports for the voxel's rows taken in ascending order; ``"first"`` the
     smallest row index; ``None`` (default) picks ``"reference"`` for grouped input and
