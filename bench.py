@@ -254,7 +254,61 @@ def frontend_timings(T, workloads, dev, N):
     k32 = keys.int()
     frontend["grid_hash_build_%dkeys_ms" % hk.numel()] = wall_ms(lambda: T.grid_hash_build(hk, hv), 20)
     frontend["grid_hash_probe_1M_ms"] = wall_ms(lambda: T.grid_hash_probe(k32, table), 20)
+    # bytes each call has to move at least (inputs read once, outputs written once), and the
+    # rate that makes at the wall-clock time above: these calls are short sequences of kernels
+    # with one or two host reads, so the rates say how far launch and latency are from mattering
+    # less than the bytes, not how well a kernel streams
+    U = int(hk.numel())
+    mb = {
+        "voxelize": N * (16 + 12 + 4),                      # xyz(+1) in; coors and keys out
+        "ScatterData_from_keys": N * (8 + 4 + 4 + 4) + U * (4 + 4 + 8 + 4),  # keys; inv, perm, seg; offsets, keys, counts, slots
+        "ingroup_inds": N * (8 + 8),
+        "grid_hash_build_%dkeys" % U: U * (4 + 4) + int(table.numel()) * 4,
+        "grid_hash_probe_1M": N * (4 + 4 + 8),              # key in, value out, at least one table slot read
+    }
+    frontend["algorithmic_MB"] = {k: round(v / 1e6, 2) for k, v in mb.items()}
+    frontend["GBps_at_wall_clock"] = {k: round(v / 1e6 / frontend[k + "_ms"], 1) for k, v in mb.items()}
     return frontend
+
+
+def frontend_cpu(workloads, N):
+    """The CPU side of the same front-end calls, once each on the host (one core unless the
+    torch op threads itself): torch.unique and the floor division as the reference's callers
+    run them, and the oracle's restatements of the other operators."""
+    import numpy as np
+    from oracle import c_oracle as orc
+    keys_cpu, key_bound = workloads._lidar_keys(N, torch.Generator().manual_seed(2))
+
+    def once_ms(fn):
+        t = time.perf_counter()
+        r = fn()
+        return (time.perf_counter() - t) * 1e3, r
+
+    out = {}
+    out["torch_unique_inverse_counts_ms"], (unq, inv, _) = once_ms(
+        lambda: torch.unique(keys_cpu, return_inverse=True, return_counts=True))
+    pts = torch.rand((N, 4), generator=torch.Generator().manual_seed(5)) * 150.0 - 75.0
+    pts[:, 2] = pts[:, 2] * (6.0 / 150.0) + 1.0
+    lo_t, vs_t = torch.tensor([-75.0, -75.0, -2.0]), torch.tensor([0.2, 0.2, 0.2])
+    out["torch_div_floor_voxelize_ms"], _ = once_ms(
+        lambda: torch.div(pts[:, :3] - lo_t[None, :], vs_t[None, :], rounding_mode="floor").int())
+    out["ingroup_inds_ms"], _ = once_ms(lambda: orc.ingroup_inds(inv.numpy()))
+    gb = torch.Generator().manual_seed(11)
+    nb = 200
+    rois = torch.zeros((nb, 7))
+    rois[:, 0:2] = torch.rand((nb, 2), generator=gb) * 140 - 70
+    rois[:, 3:6] = torch.rand((nb, 3), generator=gb) * 4 + 1
+    rois[:, 6] = torch.rand((nb,), generator=gb) * 6.283
+    p3 = pts[:200_000, :3].contiguous().numpy()
+    out["dynamic_point_pool_200boxes_200kpts_ms"], _ = once_ms(
+        lambda: orc.dynamic_point_pool(rois.numpy(), p3, [0.5, 0.5, 0.2], 512, 200_000))
+    hk = unq.numpy().astype(np.int32)
+    hv = np.arange(hk.shape[0], dtype=np.int32)
+    out["grid_hash_build_%dkeys_ms" % hk.shape[0]], table = once_ms(lambda: orc.grid_hash_build(hk, hv))
+    out["grid_hash_probe_1M_ms"], _ = once_ms(lambda: orc.grid_hash_probe(keys_cpu.numpy().astype(np.int32), table))
+    out["kind"] = "port"
+    out["sample"] = "one call each on one host core (the torch ops: torch's own threading)"
+    return out
 
 
 class KernelNames:
@@ -520,6 +574,8 @@ def main():
 
     if not a.no_cpu_baseline and a.dtype == "f32":
         out["cpu_baseline"] = cpu_baseline(w, g_mean_cpu, g_max_cpu)
+        if frontend is not None:
+            out["frontend_cpu_baseline"] = frontend_cpu(workloads, N)
     print(json.dumps(out), flush=True)
 
 
